@@ -132,9 +132,6 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
  *                            1/2 tiled kernel with that many 16-byte vectors per lane
  *   name "stereo_row_skip":   1 (default) skip the last window row when every lane of a
  *                            wavefront has an integer y (its weights are exactly 0), 0 never
- *   name "forward_sort":      1: order the queries by sampling target when a workspace is given (fp16
- *                            tiled kernels); 0 or -1 (default): natural order.  Worth switching on
- *                            for spatially incoherent 2-D offset fields only.
  *   name "forward_lds":      -1 (default) auto, 1 always, 0 never: r <= 2, head size 16/32/64 (fp16, bf16) or
  *                            16/32 (fp32), workspace given --
  *                            bucket the queries by the 16x8 tile of K/V their window centre falls in, stage

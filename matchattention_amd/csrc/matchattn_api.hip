@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void make_offsets_kernel(const T *rel, T *mo, 
     mo[(size_t)hq * 2 + 1] = Tr::from_f(cy);
 }
 
-KernelTimer g_fwd_timer = {false, nullptr, nullptr};
+KernelTimer g_fwd_timer = {{false}, nullptr, nullptr};
 
 }  // namespace ma
 
@@ -85,9 +85,17 @@ std::atomic<const char *> g_last_bwd{""};
 std::atomic<int> g_forward_variant{-1};
 std::atomic<int> g_row_skip{1};
 std::atomic<int> g_xcd_swizzle{1};
-std::atomic<int> g_forward_sort{-1};
 std::atomic<int> g_forward_lds{-1};
 std::atomic<int> g_backward_mode{-1};    // -1 auto (gather when possible), 0 scatter (atomics), 1 gather, 2 gather with the direct pass A
+
+// The options as one entry point sees them: read once per call, so that a matchattn_set_option on another thread
+// cannot make the workspace size a call checks differ from the one its kernels use.
+struct Options {
+    int forward_variant, row_skip, xcd_swizzle, forward_lds, backward_mode;
+};
+Options options_now() {
+    return Options{g_forward_variant.load(), g_row_skip.load(), g_xcd_swizzle.load(), g_forward_lds.load(), g_backward_mode.load()};
+}
 
 int fail(int code, const char *fmt, ...) {
     va_list ap;
@@ -146,7 +154,7 @@ int default_vpl(int CH, int R, int dtype) {
 
 extern "C" {
 
-int matchattn_abi_version(void) { return 3; }
+int matchattn_abi_version(void) { return 4; }
 
 const char *matchattn_last_error(void) { return g_err; }
 
@@ -178,11 +186,6 @@ int matchattn_set_option(const char *name, int value) {
         ma::g_fwd_timer.on = value != 0;
         return 0;
     }
-    if (!strcmp(name, "forward_sort")) {
-        if (value < -1 || value > 1) return fail(MATCHATTN_ERR_ARG, "matchattn_set_option: forward_sort must be -1, 0 or 1");
-        g_forward_sort = value;
-        return 0;
-    }
     return fail(MATCHATTN_ERR_ARG, "matchattn_set_option: unknown option '%s'", name);
 }
 
@@ -203,16 +206,6 @@ SortLayout sort_layout(int B, int H, int W, int h, int bin_shift = 3, int row_sh
     s.perm_off = s.rank_off + up(L * h * 4);
     s.total = s.perm_off + up(L * h * 4);
     return s;
-}
-// Whether the forward would walk the queries in target order for these sizes.
-bool sort_wanted(int B, int H, int W, int C, int h, int rx, int dtype) {
-    const int mode = g_forward_sort;
-    if (mode == 0 || dtype != MATCHATTN_F16 || rx > 2 || (int)g_forward_variant == 0) return false;
-    (void)B; (void)H; (void)W; (void)C; (void)h;
-    // auto (-1): off.  The ordering pays for spatially incoherent 2-D offset fields (-30..45 % at
-    // the optical-flow shapes) but costs 8-12 % on coherent fields, which is what a trained model
-    // produces; callers that know their field is incoherent switch it on.
-    return mode == 1;
 }
 // LDS-tile forward: buckets of the tile sort, then one flag byte per head-query (left for the generic kernel).
 struct TileLayout { SortLayout sl; size_t defer_off, chunk_off, item_off, total; int chunk_cap; };
@@ -281,9 +274,9 @@ ma::TileSort tile_sort_args(const ma::SortArgs &S, const TileLayout &tl, char *w
 }
 
 // Whether the forward would use the LDS-tile kernel for these sizes (it needs the workspace).
-bool tile_wanted(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
-    const int CH = C / h, mode = g_forward_lds;
-    if (mode == 0 || rx != ry || rx > 2 || (int)g_forward_variant == 0) return false;
+bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
+    const int CH = C / h, mode = O.forward_lds;
+    if (mode == 0 || rx != ry || rx > 2 || O.forward_variant == 0) return false;
     // head sizes with an instance (a head group is the heads that fill a 128-byte line per pixel; 64 fp32
     // channels would need 256-byte pixels: two workgroups' tiles no longer fit a CU's LDS)
     const int head_bytes = CH * (int)elem_size(dtype);
@@ -302,10 +295,15 @@ bool tile_wanted(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
 }
 }  // namespace
 
-size_t matchattn_forward_workspace_bytes(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
+namespace {
+size_t forward_workspace_bytes(const Options &O, int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
     if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || h <= 0) return 0;
-    if (tile_wanted(B, H, W, C, h, rx, ry, dtype)) return tile_layout(B, H, W, h).total;
-    return sort_wanted(B, H, W, C, h, rx, dtype) ? sort_layout(B, H, W, h).total : 0;
+    return tile_wanted(O, B, H, W, C, h, rx, ry, dtype) ? tile_layout(B, H, W, h).total : 0;
+}
+}  // namespace
+
+size_t matchattn_forward_workspace_bytes(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
+    return forward_workspace_bytes(options_now(), B, H, W, C, h, rx, ry, dtype);
 }
 
 namespace {
@@ -316,7 +314,7 @@ struct Placement {
     bool shared_offsets = false;    // every head of a pixel is known to have the same sampling position
 };
 
-int forward_impl(const void *max_offset, const void *q, const void *k, const void *v, void *out, void *attn,
+int forward_impl(const Options &O, const void *max_offset, const void *q, const void *k, const void *v, void *out, void *attn,
                  const Placement &P, void *workspace, size_t workspace_bytes,
                  int B, int H, int W, int C, int h, int rx, int ry, float scale, int dtype, void *stream) {
     if (!max_offset || !q || !k || !v || !out || !attn)
@@ -337,11 +335,11 @@ int forward_impl(const void *max_offset, const void *q, const void *k, const voi
     A.mo = max_offset; A.q = q; A.k = k; A.v = v; A.out = out; A.attn = attn;
     A.nhq = (int)(L * h); A.N = H * W; A.H = H; A.W = W; A.C = C; A.h = h;
     A.h_log2 = (h & (h - 1)) == 0 ? __builtin_ctz((unsigned)h) : -1;
-    A.scale = scale; A.row_skip = g_row_skip; A.xcd_swizzle = g_xcd_swizzle;
-    A.perm = nullptr; A.defer = nullptr;
+    A.scale = scale; A.row_skip = O.row_skip; A.xcd_swizzle = O.xcd_swizzle;
+    A.defer = nullptr;
     A.out_row_bytes = (uint32_t)(out_stride * es); A.attn_row_bytes = (uint32_t)(attn_stride * es); A.gate = P.gate;
 
-    const int variant = g_forward_variant;
+    const int variant = O.forward_variant;
     const char *kname = "";
     const void *ptrs[] = {q, k, v, out, P.gate, attn, max_offset};      // (a null gate is aligned)
     int rc = -1;
@@ -350,7 +348,7 @@ int forward_impl(const void *max_offset, const void *q, const void *k, const voi
         const int vpl = variant > 0 ? variant : default_vpl(CH, rx, dtype);
         // LDS-tile path: bucket the queries by K/V tile, one workgroup per tile and head group, then the
         // generic kernel for the (normally empty) list of queries a tile could not serve
-        if (workspace && tile_wanted(B, H, W, C, h, rx, ry, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
+        if (workspace && tile_wanted(O, B, H, W, C, h, rx, ry, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
             const TileLayout tl = tile_layout(B, H, W, h);
             const SortLayout &sl = tl.sl;
             if (workspace_bytes < tl.total)
@@ -383,19 +381,6 @@ int forward_impl(const void *max_offset, const void *q, const void *k, const voi
             if (rc != -1)
                 return fail(MATCHATTN_ERR_LAUNCH, "matchattn_forward_ws: launch of %s failed: %s", kname,
                             hipGetErrorString((hipError_t)rc));
-        }
-        // optional: order the queries by sampling target first (needs the workspace)
-        if (workspace && sort_wanted(B, H, W, C, h, rx, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
-            const SortLayout sl = sort_layout(B, H, W, h);
-            if (workspace_bytes < sl.total)
-                return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_ws: workspace of %zu bytes needed, %zu given",
-                            sl.total, workspace_bytes);
-            char *ws = (char *)workspace;
-            const ma::SortArgs S = sort_args(max_offset, dtype, B, H, W, h, sl, ws, 3, 0, 0);
-            launch_sort(S, sl, L, h, ws, false, s);
-            if (hipError_t e = hipGetLastError())
-                return fail(MATCHATTN_ERR_LAUNCH, "matchattn_forward_ws: sort launch failed: %s", hipGetErrorString(e));
-            A.perm = S.perm;
         }
         ma::timer_mark(false, s);
         switch (dtype) {
@@ -438,8 +423,8 @@ int matchattn_forward_ws(const void *max_offset, const void *q, const void *k, c
                          int B, int H, int W, int C, int h, int rx, int ry, float scale, int dtype, void *stream) {
     g_err[0] = 0;
     if (int rc = check_common("matchattn_forward", B, H, W, C, h, rx, ry, dtype)) return rc;
-    return forward_impl(max_offset, q, k, v, out, attn, Placement(), workspace, workspace_bytes, B, H, W, C, h, rx, ry, scale,
-                        dtype, stream);
+    return forward_impl(options_now(), max_offset, q, k, v, out, attn, Placement(), workspace, workspace_bytes, B, H, W, C, h, rx, ry,
+                        scale, dtype, stream);
 }
 
 float matchattn_last_forward_kernel_ms(void) {
@@ -457,7 +442,7 @@ int matchattn_forward_deferred(const void *workspace, size_t workspace_bytes,
     if (int rc = check_common("matchattn_forward_deferred", B, H, W, C, h, rx, ry, dtype)) return rc;
     if (!count) return fail(MATCHATTN_ERR_ARG, "matchattn_forward_deferred: null count pointer");
     *count = -1;
-    if (!workspace || !tile_wanted(B, H, W, C, h, rx, ry, dtype)) return MATCHATTN_OK;
+    if (!workspace || !tile_wanted(options_now(), B, H, W, C, h, rx, ry, dtype)) return MATCHATTN_OK;
     const TileLayout tl = tile_layout(B, H, W, h);
     if (workspace_bytes < tl.total)
         return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_deferred: workspace of %zu bytes needed, %zu given",
@@ -477,7 +462,7 @@ int matchattn_forward_deferred(const void *workspace, size_t workspace_bytes,
 
 size_t matchattn_forward_fused_workspace_bytes(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
     if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || h <= 0) return 0;
-    return offsets_bytes(B, H, W, h, dtype) + matchattn_forward_workspace_bytes(B, H, W, C, h, rx, ry, dtype);
+    return offsets_bytes(B, H, W, h, dtype) + forward_workspace_bytes(options_now(), B, H, W, C, h, rx, ry, dtype);
 }
 
 int matchattn_forward_fused(const void *position, int position_heads, const void *q, const void *k, const void *v,
@@ -492,16 +477,17 @@ int matchattn_forward_fused(const void *position, int position_heads, const void
                     h, position_heads);
     if (out_row_stride < 0 || attn_row_stride < 0)
         return fail(MATCHATTN_ERR_ARG, "matchattn_forward_fused: negative row stride");
+    const Options O = options_now();
     Placement P;
     P.out_stride = out_row_stride; P.attn_stride = attn_row_stride; P.gate = gate;
     P.shared_offsets = position_heads == 1;
     if (position_heads == 0)
-        return forward_impl(position, q, k, v, out, attn, P, workspace, workspace_bytes, B, H, W, C, h, rx, ry, scale, dtype, stream);
+        return forward_impl(O, position, q, k, v, out, attn, P, workspace, workspace_bytes, B, H, W, C, h, rx, ry, scale, dtype, stream);
     // relative positions: the sampling positions go to the head of the workspace, the rest serves the kernels
     const size_t ob = offsets_bytes(B, H, W, h, dtype);
     if (!workspace || workspace_bytes < ob || (reinterpret_cast<uintptr_t>(workspace) & 15u))
         return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_fused: a 16-byte aligned workspace of %zu bytes is needed, %zu given",
-                    matchattn_forward_fused_workspace_bytes(B, H, W, C, h, rx, ry, dtype), workspace ? workspace_bytes : (size_t)0);
+                    ob + forward_workspace_bytes(O, B, H, W, C, h, rx, ry, dtype), workspace ? workspace_bytes : (size_t)0);
     const int nhq = B * H * W * h;
     const float lo_x = (float)rx, hi_x = (float)((double)(W - 1 - rx) - 1e-3), lo_y = (float)ry, hi_y = (float)((double)(H - 1 - ry) - 1e-3);
     const dim3 grid((unsigned)((nhq + 255) / 256)), block(256);
@@ -523,7 +509,7 @@ int matchattn_forward_fused(const void *position, int position_heads, const void
     if (hipError_t e = hipGetLastError())
         return fail(MATCHATTN_ERR_LAUNCH, "matchattn_forward_fused: launch failed: %s", hipGetErrorString(e));
     const size_t rest = workspace_bytes - ob;
-    return forward_impl(workspace, q, k, v, out, attn, P, rest ? (char *)workspace + ob : nullptr, rest, B, H, W, C, h, rx, ry, scale,
+    return forward_impl(O, workspace, q, k, v, out, attn, P, rest ? (char *)workspace + ob : nullptr, rest, B, H, W, C, h, rx, ry, scale,
                         dtype, stream);
 }
 
@@ -531,8 +517,8 @@ namespace {
 struct BwdLayout { size_t sort_off, centre_off, dl_off, a_off, tile_off, total; SortLayout sl; bool tile; TileLayout tl; };
 // Whether pass A of the gather backward would run on LDS tiles (shapes the tile kernels have; the (dl, a)
 // scratch must fit the 32-bit offsets of a buffer descriptor).
-bool bwd_tile_wanted(int B, int H, int W, int C, int h, int rx, int dtype) {
-    const int CH = C / h, M = (2 * rx + 2) * (2 * rx + 2), mode = g_backward_mode;
+bool bwd_tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
+    const int CH = C / h, M = (2 * rx + 2) * (2 * rx + 2), mode = O.backward_mode;
     if (mode == 2 || mode == 0) return false;
     const int head_bytes = CH * (int)elem_size(dtype);
     if (!(rx <= 2 && (CH == 16 || CH == 32 || (CH == 64 && dtype != MATCHATTN_F32)) &&
@@ -541,7 +527,7 @@ bool bwd_tile_wanted(int B, int H, int W, int C, int h, int rx, int dtype) {
         return false;
     return mode == 1 || (long long)B * H * W * h >= (1ll << 18);   // auto: maps large enough to pay for the bucketing
 }
-BwdLayout bwd_gather_layout(int B, int H, int W, int C, int h, int rx, int dtype) {
+BwdLayout bwd_gather_layout(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
     BwdLayout l;
     l.sl = sort_layout(B, H, W, h, 0);              // one bin per target pixel
     const size_t nhq = (size_t)B * H * W * h, M = (size_t)(2 * rx + 2) * (2 * rx + 2);
@@ -552,7 +538,7 @@ BwdLayout bwd_gather_layout(int B, int H, int W, int C, int h, int rx, int dtype
     l.a_off = l.dl_off + up(nhq * M * 4);
     l.tile_off = l.a_off + up(nhq * M * 4);
     l.total = l.tile_off;
-    l.tile = bwd_tile_wanted(B, H, W, C, h, rx, dtype);
+    l.tile = bwd_tile_wanted(O, B, H, W, C, h, rx, dtype);
     if (l.tile) {
         l.tl = tile_layout(B, H, W, h);
         l.total += up(l.tl.total);
@@ -564,8 +550,8 @@ size_t bwd_scatter_bytes(int B, int H, int W, int C, int dtype) {
     const size_t n = (size_t)B * H * W * C;
     return 2 * (((n * sizeof(float)) + 255) & ~(size_t)255);
 }
-bool bwd_gather_possible(int B, int H, int W, int C, int h, int rx, int dtype) {
-    if (g_backward_mode == 0 || (int)g_forward_variant == 0 || C % h) return false;
+bool bwd_gather_possible(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
+    if (O.backward_mode == 0 || O.forward_variant == 0 || C % h) return false;
     const int CH = C / h;
     const long long L = (long long)B * H * W;
     return bwd_tiled_shape(CH, rx, dtype) && (CH * elem_size(dtype)) % 16 == 0 && H < 30000 && W < 30000 &&
@@ -573,15 +559,21 @@ bool bwd_gather_possible(int B, int H, int W, int C, int h, int rx, int dtype) {
 }
 }  // namespace
 
-size_t matchattn_backward_workspace_bytes(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
-    (void)ry;
+namespace {
+size_t backward_workspace_bytes(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
     if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || h <= 0) return 0;
     size_t need = bwd_scatter_bytes(B, H, W, C, dtype);
-    if (bwd_gather_possible(B, H, W, C, h, rx, dtype)) {
-        const size_t g = bwd_gather_layout(B, H, W, C, h, rx, dtype).total;
+    if (bwd_gather_possible(O, B, H, W, C, h, rx, dtype)) {
+        const size_t g = bwd_gather_layout(O, B, H, W, C, h, rx, dtype).total;
         if (g > need) need = g;
     }
     return need;
+}
+}  // namespace
+
+size_t matchattn_backward_workspace_bytes(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
+    (void)ry;
+    return backward_workspace_bytes(options_now(), B, H, W, C, h, rx, dtype);
 }
 
 int matchattn_backward(const void *max_offset, const void *q, const void *k, const void *v, const void *d_out,
@@ -592,7 +584,8 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
     if (int rc = check_common("matchattn_backward", B, H, W, C, h, rx, ry, dtype)) return rc;
     if (!max_offset || !q || !k || !v || !d_out || !dq || !dk || !dv || !d_max_offset)
         return fail(MATCHATTN_ERR_ARG, "matchattn_backward: null tensor pointer");
-    const size_t need = matchattn_backward_workspace_bytes(B, H, W, C, h, rx, ry, dtype);
+    const Options O = options_now();
+    const size_t need = backward_workspace_bytes(O, B, H, W, C, h, rx, dtype);
     if (need && (!workspace || workspace_bytes < need))
         return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_backward: workspace of %zu bytes needed, %zu given", need,
                     workspace ? workspace_bytes : (size_t)0);
@@ -610,14 +603,14 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
     A.perm = nullptr; A.centre = nullptr; A.bin_start = nullptr; A.row_start = nullptr; A.per_head = nullptr; A.nrows = B * H;
     A.only_flagged = nullptr;
     A.nhq = (int)(L * h); A.N = H * W; A.H = H; A.W = W; A.C = C; A.h = h;
-    A.scale = scale; A.xcd_swizzle = g_xcd_swizzle;
+    A.scale = scale; A.xcd_swizzle = O.xcd_swizzle;
 
     // ---- gather mode: deterministic, no atomics (pass A per query, inverse index, pass B per key) ----
     {
         const void *gp[] = {q, k, v, d_out, dq, dk, dv};
-        if (bwd_gather_possible(B, H, W, C, h, rx, dtype) && tiled_ok(gp, 7, L, C, CH, dtype) &&
+        if (bwd_gather_possible(O, B, H, W, C, h, rx, dtype) && tiled_ok(gp, 7, L, C, CH, dtype) &&
             (!d_attn || (reinterpret_cast<uintptr_t>(d_attn) & (elem_size(dtype) - 1)) == 0)) {
-            const BwdLayout bl = bwd_gather_layout(B, H, W, C, h, rx, dtype);
+            const BwdLayout bl = bwd_gather_layout(O, B, H, W, C, h, rx, dtype);
             if (!workspace || workspace_bytes < bl.total)
                 return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_backward: workspace of %zu bytes needed, %zu given",
                             bl.total, workspace ? workspace_bytes : (size_t)0);
@@ -701,7 +694,7 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
     const void *ptrs[] = {q, k, v, d_out, dq};
     const char *kname = "";
     int rc = -1;
-    if ((int)g_forward_variant != 0 && rx <= 2 && tiled_ok(ptrs, 5, L, C, CH, dtype) &&
+    if (O.forward_variant != 0 && rx <= 2 && tiled_ok(ptrs, 5, L, C, CH, dtype) &&
         (!d_attn || (reinterpret_cast<uintptr_t>(d_attn) & (elem_size(dtype) - 1)) == 0)) {
         switch (dtype) {
         case MATCHATTN_F32: rc = ma::launch_bwd_tiled_f32(A, CH, rx, s, &kname); break;

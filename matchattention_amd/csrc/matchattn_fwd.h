@@ -19,7 +19,6 @@ struct FwdArgs {
     int hpg_log2; // fp16 kernel: log2 of the heads per block group (a power of two dividing h)
     float scale;
     int row_skip; // allow skipping the last window row when every lane has integer y
-    const int *perm;      // fp16 kernel: optional [h][B*N] processing order (pixel indices per head), or null
     int xcd_swizzle;
     const uint8_t *defer; // generic kernel: optional [nhq] flags, compute only the head-queries whose flag is set; or null
     // Output placement.  `out` holds one row of C values per pixel every out_row_bytes, `attn` one row of h*M

@@ -71,10 +71,7 @@ __global__ __launch_bounds__(256, h16_waves(R, VPL)) void fwd_h16_kernel(FwdArgs
     const int head = hgrp * hpg + (grp & (hpg - 1));
     const bool tail = slot >= npix;          // whole lane groups fall off the end together
     if (tail) slot = npix - 1;               // keep them in flight (DPP partners), store nothing
-    // slots are pixels in natural order, or in the order of the target sort (matchattn_sort.h)
-    // (a complete permutation per head; the entry is clamped so that no value read from the
-    // scratch buffer can turn into an out-of-range address)
-    const int pix = A.perm ? clampi(A.perm[(size_t)head * npix + slot], 0, npix - 1) : slot;
+    const int pix = slot;
     const int hq = pix * A.h + head;
     const bool carries = sub < Cfg::NVL;
     const bool live = carries && !tail;

@@ -3,6 +3,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 namespace ma {
 
 struct FwdArgs;
@@ -27,7 +29,7 @@ int launch_fwd_tile_bf16(const FwdArgs &A, const TileSort &S, int CH, int R, hip
 
 // Optional timing of the dominant kernel of a forward call (option "time_kernels"): when `on`, the launcher of
 // that kernel records the two events on the stream either side of the launch.
-struct KernelTimer { bool on; hipEvent_t before, after; };
+struct KernelTimer { std::atomic<bool> on; hipEvent_t before, after; };
 extern KernelTimer g_fwd_timer;
 inline void timer_mark(bool end, hipStream_t s) {
     if (g_fwd_timer.on) (void)hipEventRecord(end ? g_fwd_timer.after : g_fwd_timer.before, s);

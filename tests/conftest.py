@@ -20,3 +20,18 @@ def hip_lib():
         pytest.skip("no GPU visible")
     from matchattention_amd import _cabi
     return _cabi.load()
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Worst measured error per label of every tests.util.check_err call, with its bound."""
+    from tests import util
+    if not util.MEASURED:
+        return
+    worst = {}
+    for label, err, tol in util.MEASURED:
+        if label not in worst or err / tol > worst[label][0] / worst[label][1]:
+            worst[label] = (err, tol)
+    terminalreporter.write_sep("-", "measured errors (max|a-b| / max|b|), worst per label")
+    for label in sorted(worst):
+        err, tol = worst[label]
+        terminalreporter.write_line(f"{label:60s} {err:9.3e}  bound {tol:.1e}  ({err / tol:5.2f} x)")

@@ -11,11 +11,9 @@ import torch
 from oracle import mat_oracle as O
 from tests.gpu_util import hip_backward, hip_forward
 from tests.test_oracle_golden import GOLDEN, load_golden
-from tests.util import make_case, rel_err
+from tests.util import GRAD_TOL, GRAD_TOL_GOLDEN, TOL, check_err, check_grads, make_case, rel_err
 
 pytestmark = pytest.mark.gpu
-
-TOL = {torch.float32: 1e-5, torch.float16: 2e-3, torch.bfloat16: 2e-2}
 
 
 def _dev(*ts):
@@ -37,11 +35,10 @@ def test_backward_matches_reference_golden(hip_lib, path):
     g = load_golden(path)
     mo, q, k, v, d_out, d_attn = _dev(g["max_offset"], g["q"], g["k"], g["v"], g["d_out"], g["d_attn"])
     grads = hip_backward(hip_lib, mo, q, k, v, g["H"], g["W"], g["r"], g["Ch"] ** -0.5, d_out, d_attn)
-    # The reference's gradients are themselves autograd in the tensor dtype (half-precision
-    # scatter-adds); the kernel accumulates in fp32, so allow the reference's own rounding noise.
-    tol = {torch.float32: 2e-5, torch.float16: 6e-3, torch.bfloat16: 5e-2}[g["dtype"]]
+    # (the reference's gradients are themselves autograd in the tensor dtype)
+    dtn = str(g["dtype"]).split(".")[1]
     for got, name in zip(grads, ("dq", "dk", "dv", "dmo")):
-        assert rel_err(got.cpu(), g[name]) <= tol, name
+        check_err(got.cpu(), g[name], GRAD_TOL_GOLDEN[g["dtype"]], f"golden bwd {name} {dtn}")
 
 
 CASES = [
@@ -84,12 +81,8 @@ def test_forward_and_backward_match_oracle(hip_lib, case):
     M = (2 * r + 2) ** 2
     d_out = torch.randn(B, H * W, h * Ch, generator=g).to(dt)
     d_attn = torch.randn(B, H * W, h, M, generator=g).to(dt)
-    want = O.backward(mo.double(), q.double(), k.double(), v.double(), H, W, [r, r], scale, d_out.double(), d_attn.double())
     got = hip_backward(hip_lib, dmo_, dq_, dk_, dv_, H, W, r, scale, d_out.cuda(), d_attn.cuda())
-    gtol = {torch.float32: 2e-5, torch.float16: 4e-3, torch.bfloat16: 4e-2}[dt]
-    for a, b, name in zip(got, want, ("dq", "dk", "dv", "dmo")):
-        assert torch.isfinite(a).all(), name
-        assert rel_err(a.cpu(), b) <= gtol, name
+    check_grads(got, mo, q, k, v, H, W, r, scale, d_out, d_attn, "seeded cases bwd")
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2])
@@ -104,7 +97,6 @@ def test_both_backward_modes_agree_with_autograd(hip_lib, mode, dt, offs, clamp,
     g = torch.Generator().manual_seed(3)
     d_out = torch.randn(B, H * W, h * Ch, generator=g).to(dt)
     d_attn = torch.randn(B, H * W, h, 36, generator=g).to(dt)
-    want = O.backward(mo.double(), q.double(), k.double(), v.double(), H, W, [r, r], 0.2, d_out.double(), d_attn.double())
     try:
         _cabi.set_option("backward_mode", mode)
         got = hip_backward(hip_lib, *_dev(mo, q, k, v), H, W, r, 0.2, d_out.cuda(), d_attn.cuda())
@@ -113,10 +105,7 @@ def test_both_backward_modes_agree_with_autograd(hip_lib, mode, dt, offs, clamp,
             assert all(torch.equal(a, b) for a, b in zip(got, again))
     finally:
         _cabi.set_option("backward_mode", -1)
-    tol = 2e-5 if dt == torch.float32 else 4e-3
-    for a, b, name in zip(got, want, ("dq", "dk", "dv", "dmo")):
-        assert torch.isfinite(a).all(), name
-        assert rel_err(a.cpu(), b) <= tol, (name, mode)
+    check_grads(got, mo, q, k, v, H, W, r, 0.2, d_out, d_attn, f"backward_mode {mode} bwd")
 
 
 @pytest.mark.parametrize("offs,per_head,clamp,Ch,r,shape,with_dattn", [
@@ -137,8 +126,6 @@ def test_lds_tile_backward_matches_autograd(hip_lib, dt, offs, per_head, clamp, 
     d_out = torch.randn(B, H * W, h * Ch, generator=g).to(dt)
     d_attn = torch.randn(B, H * W, h, M, generator=g).to(dt) if with_dattn else None
     scale = Ch ** -0.5
-    want = O.backward(mo.double(), q.double(), k.double(), v.double(), H, W, [r, r], scale, d_out.double(),
-                      d_attn.double() if with_dattn else None)
     dev = _dev(mo, q, k, v)
     try:
         _cabi.set_option("backward_mode", 1)
@@ -150,22 +137,18 @@ def test_lds_tile_backward_matches_autograd(hip_lib, dt, offs, per_head, clamp, 
     finally:
         _cabi.set_option("backward_mode", -1)
     assert name == "bwd_tile_" + {torch.float16: "f16", torch.float32: "f32", torch.bfloat16: "bf16"}[dt], name
-    gtol = {torch.float32: 2e-5, torch.float16: 4e-3, torch.bfloat16: 4e-2}[dt]
-    for a, b, c, d, nm in zip(got, want, again, direct, ("dq", "dk", "dv", "dmo")):
-        assert torch.isfinite(a).all(), nm
-        assert rel_err(a.cpu(), b) <= gtol, nm
+    check_grads(got, mo, q, k, v, H, W, r, scale, d_out, d_attn, "lds-tile bwd")
+    for a, c, d, nm in zip(got, again, direct, ("dq", "dk", "dv", "dmo")):
         assert torch.equal(a, c), nm                          # bucket order does not change a result
-        assert rel_err(a.cpu(), d.cpu().double()) <= gtol / 2, nm     # the two pass-A kernels agree
+        assert rel_err(a.cpu(), d.cpu().double()) <= TOL[dt], nm     # the two pass-A kernels agree
 
 
 def test_backward_without_attention_gradient(hip_lib):
     B, H, W, h, Ch, r = 1, 9, 10, 2, 32, 2
     mo, q, k, v = make_case(B, H, W, h, Ch, r, torch.float32, seed=5)
     d_out = torch.randn(B, H * W, h * Ch, generator=torch.Generator().manual_seed(1))
-    want = O.backward(mo, q, k, v, H, W, [r, r], 0.2, d_out, None)
     got = hip_backward(hip_lib, *_dev(mo, q, k, v), H, W, r, 0.2, d_out.cuda(), None)
-    for a, b, name in zip(got, want, ("dq", "dk", "dv", "dmo")):
-        assert rel_err(a.cpu(), b) <= 2e-5, name
+    check_grads(got, mo, q, k, v, H, W, r, 0.2, d_out, None, "no-dattn bwd")
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2])
@@ -200,27 +183,6 @@ def test_row_skip_does_not_change_results(hip_lib):
     assert rel_err(out0, out1) <= 1e-3 and rel_err(attn0, attn1) <= 1e-3
     a = attn1.view(B, H * W, h, 2 * r + 2, 2 * r + 2)
     assert (a[..., -1, :] == 0).all()          # integer y: the last window row has weight exactly 0
-
-
-@pytest.mark.parametrize("offs,per_head", [("stereo", False), ("mixed", True), ("mixed", False)])
-def test_target_ordered_forward_is_identical(hip_lib, offs, per_head):
-    # forward_sort=1 walks the queries in the order of a counting sort on their sampling targets
-    from matchattention_amd import _cabi
-    B, H, W, h, Ch, r = 2, 21, 37, 4, 32, 2
-    mo, q, k, v = make_case(B, H, W, h, Ch, r, torch.float16, seed=55, offsets=offs, per_head=per_head)
-    args = _dev(mo, q, k, v)
-    try:
-        _cabi.set_option("forward_sort", 0)
-        out0, attn0 = hip_forward(hip_lib, *args, H, W, r, Ch ** -0.5)
-        _cabi.set_option("forward_sort", 1)
-        assert hip_lib.matchattn_forward_workspace_bytes(B, H, W, h * Ch, h, r, r, 1) > 0
-        out1, attn1 = hip_forward(hip_lib, *args, H, W, r, Ch ** -0.5)
-    finally:
-        _cabi.set_option("forward_sort", -1)
-    # row skip is decided per wavefront, which the order changes: a final rounding may differ
-    assert rel_err(attn0, attn1) <= 1e-3 and rel_err(out0, out1) <= 1e-3
-    want_out, want_attn = O.forward(mo, q, k, v, H, W, [r, r], Ch ** -0.5)
-    assert rel_err(attn1.cpu(), want_attn) <= 2e-3 and rel_err(out1.cpu(), want_out) <= 2e-3
 
 
 @pytest.mark.parametrize("offs,per_head,clamp,Ch,r,shape", [
@@ -591,8 +553,6 @@ def test_random_shapes_match_oracle(hip_lib, case):
     d_out = torch.randn(B, H * W, h * Ch, generator=g).to(dt)
     d_attn = torch.randn(B, H * W, h, M, generator=g).to(dt) if idx % 3 else None
     want_out, want_attn = O.forward(mo, q, k, v, H, W, [r, r], scale)
-    want = O.backward(mo.double(), q.double(), k.double(), v.double(), H, W, [r, r], scale, d_out.double(),
-                      None if d_attn is None else d_attn.double())
     dev = _dev(mo, q, k, v)
     try:
         _cabi.set_option("forward_lds", lds)
@@ -605,10 +565,7 @@ def test_random_shapes_match_oracle(hip_lib, case):
     tol = TOL[dt]
     assert torch.isfinite(out).all() and torch.isfinite(attn).all()
     assert rel_err(attn.cpu(), want_attn) <= tol and rel_err(out.cpu(), want_out) <= tol
-    gtol = {torch.float32: 2e-5, torch.float16: 4e-3, torch.bfloat16: 4e-2}[dt]
-    for a, b, name in zip(got, want, ("dq", "dk", "dv", "dmo")):
-        assert torch.isfinite(a).all(), name
-        assert rel_err(a.cpu(), b) <= gtol, (name, _cabi.last_backward_kernel())
+    check_grads(got, mo, q, k, v, H, W, r, scale, d_out, d_attn, "random shapes bwd")
 
 
 @pytest.mark.parametrize("tiles", [False, True])
@@ -732,4 +689,4 @@ def test_misaligned_tensors_take_the_generic_kernels(hip_lib):
     torch.cuda.synchronize()
     assert _cabi.last_backward_kernel().startswith("bwd_generic")
     for got, want in zip((out, attn, dq, dk, dv, dmo), want_f + want_b):
-        assert rel_err(got.float().cpu(), want.float().cpu()) <= 4e-3
+        assert rel_err(got.float().cpu(), want.float().cpu()) <= 2e-3

@@ -26,7 +26,7 @@ def test_module_forward_and_autograd(hip_lib):
     assert rel_err(out.detach().cpu(), out_r.detach()) <= 1e-5
     assert rel_err(attn.detach().cpu(), attn_r.detach()) <= 1e-5
     for a, b in zip(dev_in, ref_in):
-        assert rel_err(a.grad.cpu(), b.grad) <= 5e-5
+        assert rel_err(a.grad.cpu(), b.grad) <= 1e-5
     # inference path (no grad): in-place opaque op, same numbers
     with torch.no_grad():
         out2, attn2 = op(*[t.detach() for t in dev_in], H, W, [r, r], 36, "l1_norm", scale)

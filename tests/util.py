@@ -39,3 +39,43 @@ def rel_err(a: torch.Tensor, b: torch.Tensor) -> float:
     """max |a-b| / max |b|  -- the norm-wise relative error the tolerances refer to."""
     a, b = a.double(), b.double()
     return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+# Every comparison made through check_err is kept, and the session's summary (tests/conftest.py) prints the
+# worst measured error per label beside its bound, so that a run shows how far each bound is from binding.
+MEASURED = []
+
+
+def check_err(got: torch.Tensor, want: torch.Tensor, tol: float, label: str) -> float:
+    """Asserts rel_err(got, want) <= tol and records the measured value under `label`."""
+    e = rel_err(got, want)
+    MEASURED.append((label, e, tol))
+    assert e <= tol, f"{label}: {e:.3e} > {tol:.1e}"
+    return e
+
+
+# Bounds of the comparisons (same metric everywhere): 1e-5 in fp32 and 2e-3 in fp16 as the operator's parity
+# target states them, 2e-2 in bf16 (8 significand bits instead of 11).
+TOL = {torch.float32: 1e-5, torch.float16: 2e-3, torch.bfloat16: 2e-2}
+# Gradients at full size (hundreds of contributions per element, errors average out) and against the reference's
+# own gradients (the golden vectors) take the same bounds.
+GRAD_TOL = TOL
+GRAD_TOL_GOLDEN = TOL
+
+
+def check_grads(got, mo, q, k, v, H, W, r, scale, d_out, d_attn, label):
+    """Gradients of a small case against the exact gradient (the oracle's autograd in fp64 on the same rounded
+    inputs).  fp32: within 1e-5.  16-bit types: the definition's own gradient in that type (autograd through
+    half-precision gathers, products and scatter-adds) lies up to 9e-3 (fp16) from the exact one on maps this
+    small (tests/test_oracle_math.py measures it), and the parity target is stated against the definition: a
+    gradient within `tol` of the definition's lies within `tol + |definition - exact|` of the exact one, which is
+    the bound per tensor here, with the second term measured on this very case.  (The kernel accumulates in
+    fp32; comparing it with the definition's fp16 sums directly would test the reference's noise, not the kernel.)"""
+    dt = q.dtype
+    dbl = lambda t: None if t is None else t.double()
+    exact = O.backward(dbl(mo), dbl(q), dbl(k), dbl(v), H, W, [r, r], scale, dbl(d_out), dbl(d_attn))
+    own = exact if dt == torch.float32 else O.backward(mo, q, k, v, H, W, [r, r], scale, d_out, d_attn)
+    name = str(dt).split(".")[1]
+    for a, b, c, tensor in zip(got, exact, own, ("dq", "dk", "dv", "dmo")):
+        assert torch.isfinite(a).all(), tensor
+        check_err(a.cpu(), b, TOL[dt] + rel_err(c, b), f"{label} {tensor} {name}")
