@@ -75,6 +75,24 @@ int matchattn_forward_ws(const void *max_offset, const void *q, const void *k, c
                          float scale, int dtype, void *stream);
 
 /*
+ * matchattn_forward_ws on scratch memory the library owns.  No counterpart in the reference: it is for callers
+ * that cannot allocate device memory around the call -- code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  The scratch is one static device array of matchattn_static_scratch_bytes()
+ * = 40 MiB per GPU (held by every GPU the library is used on until the process ends), enough for 4.6 M
+ * head-queries (B*H*W*h; the 544x960, 8-head map needs 36.2 MiB); larger sizes are rejected with
+ * MATCHATTN_ERR_WORKSPACE.  Neither call allocates or frees anything; results are bit-identical to
+ * matchattn_forward_ws.  Every call on a GPU uses that GPU's one array, so two calls that overlap on one GPU
+ * (two streams, two threads) race: serialise them.  matchattn_static_scratch_bytes looks the array's device
+ * address up for the current device (once per device; matchattn_forward_static does the same on its first call
+ * there) and returns the capacity, or 0 with the error set: call it once per device before a stream capture.
+ */
+size_t matchattn_static_scratch_bytes(void);
+int matchattn_forward_static(const void *max_offset, const void *q, const void *k, const void *v,
+                             void *out, void *attn,
+                             int B, int H, int W, int C, int h, int rx, int ry,
+                             float scale, int dtype, void *stream);
+
+/*
  * Forward fused with the steps the attention module runs either side of the operator.
  *
  * Before (replaces the elementwise passes of models/attention_blocks.py:149-151 / 162-163 and the module's

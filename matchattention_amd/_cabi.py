@@ -21,6 +21,8 @@ SIGNATURES = {
     "matchattn_forward": (_i, [_vp] * 6 + [_i] * 7 + [_f, _i, _vp]),
     "matchattn_forward_workspace_bytes": (_sz, [_i] * 8),
     "matchattn_forward_ws": (_i, [_vp] * 7 + [_sz] + [_i] * 7 + [_f, _i, _vp]),
+    "matchattn_static_scratch_bytes": (_sz, []),
+    "matchattn_forward_static": (_i, [_vp] * 6 + [_i] * 7 + [_f, _i, _vp]),
     "matchattn_forward_fused_workspace_bytes": (_sz, [_i] * 8),
     "matchattn_forward_fused": (_i, [_vp, _i] + [_vp] * 5 + [_ll, _vp, _ll, _vp, _sz] + [_i] * 7 + [_f, _i, _vp]),
     "matchattn_backward_workspace_bytes": (_sz, [_i] * 8),

@@ -427,6 +427,72 @@ int matchattn_forward_ws(const void *max_offset, const void *q, const void *k, c
                         scale, dtype, stream);
 }
 
+// ---- forward on the library's own scratch: nothing is allocated by the caller or by the call ------------------
+// One array per GPU (each device that loads the library holds its own copy at its own address, until the process
+// ends).  In host code the array's name is only a handle for hipGetSymbolAddress: kernels, fills and copies take
+// the device address that call returns, kept per device below.
+}  // extern "C"
+
+namespace {
+constexpr size_t kStaticScratchBytes = (size_t)40 << 20;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+namespace {
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up once per device), or null with the error set.
+void *static_scratch(const char *fn) {
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev)) {
+        fail(MATCHATTN_ERR_LAUNCH, "%s: hipGetDevice failed: %s", fn, hipGetErrorString(e));
+        return nullptr;
+    }
+    if (dev < 0 || dev >= kMaxDevices) {
+        fail(MATCHATTN_ERR_ARG, "%s: device index %d beyond the %d this entry point keeps scratch for", fn, dev, kMaxDevices);
+        return nullptr;
+    }
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) {
+        fail(MATCHATTN_ERR_LAUNCH, "%s: hipGetSymbolAddress failed on device %d: %s", fn, dev, hipGetErrorString(e));
+        return nullptr;
+    }
+    if (!p || (reinterpret_cast<uintptr_t>(p) & 255u)) {
+        fail(MATCHATTN_ERR_LAUNCH, "%s: scratch array at %p on device %d is not 256-byte aligned", fn, p, dev);
+        return nullptr;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // (two threads racing here store the same address)
+    return p;
+}
+}  // namespace
+
+extern "C" {
+
+size_t matchattn_static_scratch_bytes(void) {
+    g_err[0] = 0;
+    return static_scratch("matchattn_static_scratch_bytes") ? kStaticScratchBytes : 0;
+}
+
+int matchattn_forward_static(const void *max_offset, const void *q, const void *k, const void *v, void *out, void *attn,
+                             int B, int H, int W, int C, int h, int rx, int ry, float scale, int dtype, void *stream) {
+    g_err[0] = 0;
+    if (int rc = check_common("matchattn_forward_static", B, H, W, C, h, rx, ry, dtype)) return rc;
+    const Options O = options_now();
+    const size_t need = forward_workspace_bytes(O, B, H, W, C, h, rx, ry, dtype);
+    if (need > kStaticScratchBytes)
+        return fail(MATCHATTN_ERR_WORKSPACE,
+                    "matchattn_forward_static: these sizes need %zu bytes of scratch, the library's own array holds %zu "
+                    "(B*H*W*h = %lld head-queries; use matchattn_forward_ws with a caller-provided workspace)",
+                    need, kStaticScratchBytes, (long long)B * H * W * h);
+    void *ws = nullptr;
+    if (need) {
+        ws = static_scratch("matchattn_forward_static");
+        if (!ws) return MATCHATTN_ERR_LAUNCH;
+    }
+    return forward_impl(O, max_offset, q, k, v, out, attn, Placement(), ws, need, B, H, W, C, h, rx, ry, scale, dtype, stream);
+}
+
 float matchattn_last_forward_kernel_ms(void) {
     if (!ma::g_fwd_timer.on || !ma::g_fwd_timer.after) return -1.f;
     float ms = -1.f;
