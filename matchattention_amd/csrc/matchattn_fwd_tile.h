@@ -87,8 +87,29 @@ __device__ __forceinline__ void bucket_bounds(const TileSort &S, int src, int bi
     hi = clampi(hi, lo, S.L);
 }
 
-// chunk_start[bin] = number of chunks in the buckets before `bin` (exclusive scan), chunk_start[nbins] =
-// all of them; chunk_item[c] = (bucket, index within the bucket) of chunk c.  A bucket has ceil(n / kTileCap) chunks, n being its largest population over the heads;
+// Order in which the work list visits the tiles of an image: strips of kTileStrip tile columns, each walked row by
+// row from the top.  The workgroups of an XCD take consecutive items, so the tiles in flight form a block about as
+// tall as it is wide and the K/V rows a tile shares with the tile below it are still in that XCD's L2 when the
+// tile below is staged (in row-major order a whole tile row -- more than the L2 holds, with the query, output
+// and attention streams of its items -- passes in between, and the vertical halo is fetched from memory again).
+#ifndef MA_TILE_STRIP
+#define MA_TILE_STRIP 8
+#endif
+constexpr int kTileStrip = MA_TILE_STRIP;
+__device__ __forceinline__ int tile_visit_order(const TileSort &S, int k) {
+    if (kTileStrip <= 0 || S.bins_per_row <= kTileStrip) return k;
+    const int per_img = S.rows_per_img * S.bins_per_row;
+    const int img = k / per_img, kk = k - img * per_img;
+    const int nfull = S.bins_per_row / kTileStrip;
+    const int strip = min(kk / (S.rows_per_img * kTileStrip), nfull);
+    const int w = strip < nfull ? kTileStrip : S.bins_per_row - nfull * kTileStrip;
+    const int within = kk - strip * S.rows_per_img * kTileStrip;
+    const int r = within / w, c = strip * kTileStrip + (within - r * w);
+    return (img * S.rows_per_img + r) * S.bins_per_row + c;
+}
+
+// chunk_start[bin] = number of chunks in the buckets visited before `bin` (exclusive scan in visiting order),
+// chunk_start[nbins] = all of them; chunk_item[c] = (bucket, index within the bucket) of chunk c.  A bucket has ceil(n / kTileCap) chunks, n being its largest population over the heads;
 // empty buckets have none.  One workgroup of 1024 threads.
 template <int Unused = 0>   // a template only so that several translation units may include this header
 __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, int *chunk_start) {
@@ -97,7 +118,8 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
     const int b0 = min((int)threadIdx.x * per, S.nbins), b1 = min(b0 + per, S.nbins);
     const int nh = *S.per_head ? h : 1;
     int sum = 0;
-    for (int bin = b0; bin < b1; ++bin) {
+    for (int pos = b0; pos < b1; ++pos) {
+        const int bin = tile_visit_order(S, pos);
         int n = 0;
         for (int hd = 0; hd < nh; ++hd) {
             int lo, hi;
@@ -117,7 +139,8 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
         __syncthreads();
     }
     int run = part[threadIdx.x] - sum;
-    for (int bin = b0; bin < b1; ++bin) {
+    for (int pos = b0; pos < b1; ++pos) {
+        const int bin = tile_visit_order(S, pos);
         const int c = chunk_start[bin];
         chunk_start[bin] = run;
         // the work list itself: entry = (bucket, which chunk of it), so that a workgroup finds its item with one load
@@ -150,9 +173,22 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     const __amdgpu_buffer_rsrc_t rgate = make_rsrc(A.gate, A.gate ? total_bytes : 0u);   // (no gate: every load is out of range)
     const __amdgpu_buffer_rsrc_t rm = make_rsrc(A.mo, (uint32_t)A.nhq * 4u);
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(S.defer, (uint32_t)A.nhq);
-    const int sub = threadIdx.x % LPH;
-    const int grp = threadIdx.x / LPH;
+    // With two lanes per head-query the pair is lanes l and l ^ 16 of a wavefront (not neighbours): the sum of a
+    // tap's |q - k| over the pair's 32 channels is then what one matrix instruction delivers to both lanes
+    // (see pair_ones below), and the vector ALU is left with the subtractions and the sign masks.
+    constexpr bool kMatrixSum = LPH == 2 && VPL == 2;
+    const int lane_w = threadIdx.x & 63;
+    const int sub = kMatrixSum ? ((lane_w >> 4) & 1) : (int)(threadIdx.x % LPH);
+    const int grp = kMatrixSum ? (int)(threadIdx.x >> 6) * 32 + (lane_w & 15) + ((lane_w >> 5) << 4) : (int)(threadIdx.x / LPH);
     const int hslot = grp % HPG, gi = grp / HPG;
+    // A operand of v_mfma_f32_16x16x32_f16 (16 x 32, lane i + 16 (k / 8) holds A[i][k..k+7]) that is 1 where row i and
+    // column block k / 8 belong to the same half of the wavefront's four 16-lane blocks and 0 elsewhere: with the
+    // |q - k| halves as the B operand (lane j + 16 b holds column j, rows 8 b .. 8 b + 7) every lane receives, in each
+    // of its four result registers, the sum over the 8 halves of lanes l and l ^ 16.
+    typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    const uint32_t one_bits = (((lane_w & 15) >= 8) == (lane_w >= 32)) ? 0x3c003c00u : 0u;
+    [[maybe_unused]] const half8_t pair_ones = __builtin_bit_cast(half8_t, u32x4{one_bits, one_bits, one_bits, one_bits});
     // Lane `sub` owns the 16-byte vectors sub, sub + LPH, ... of its head, so that the lanes of one LDS read
     // touch adjacent 16-byte pieces (vectors 2 sub, 2 sub + 1 would put them 32 bytes apart: 2-way bank
     // conflicts).  With two vectors per lane, odd lane groups take theirs in the opposite order: one LDS
@@ -171,6 +207,11 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     // (MA_TILE_QUEUE; a fixed stride without it).
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
     const int nitems = nchunks * nhg;
+    // Item -> (chunk, head group).  The head groups of a chunk are neighbours in the list: the items an XCD has in
+    // flight then cover whole pixel rows of a block of tiles.  (With the head group as the slow index an XCD would
+    // touch one 128-byte line in every 128 * nhg bytes, which its L2 maps to a fraction of its sets.)
+    auto item_chunk = [&](int it) __attribute__((always_inline)) { return it / nhg; };
+    auto item_hgrp = [&](int it) __attribute__((always_inline)) { return it - (it / nhg) * nhg; };
     const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
     const int item_end = (int)((long long)nitems * (xcd + 1) >> 3);
     const bool per_head = *S.per_head != 0;
@@ -195,7 +236,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     const int item0 = (int)((long long)nitems * xcd >> 3) + (int)(blockIdx.x >> 3);
 #endif
     int2 entry = int2{0, 0};
-    if (item0 < item_end) entry = S.chunk_item[item0 - (item0 / nchunks) * nchunks];
+    if (item0 < item_end) entry = S.chunk_item[item_chunk(item0)];
 #if MA_TILE_QUEUE
     for (int item = item0; item < item_end;) {
     int claim = 0;
@@ -203,7 +244,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #else
     for (int item = item0; item < item_end; item += per_xcd) {
 #endif
-    const int hgrp = item / nchunks;
+    const int hgrp = item_hgrp(item);
     const int bin = clampi(entry.x, 0, S.nbins - 1), part = max(entry.y, 0);
     // this lane group's head and its share of the bucket
     const int head = hgrp * HPG + hslot;
@@ -258,7 +299,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #else
     const int item_n = min(item + per_xcd, item_end - 1);       // (the last item fetches its own entry again)
 #endif
-    const int2 entry_n = S.chunk_item[item_n - (item_n / nchunks) * nchunks];
+    const int2 entry_n = S.chunk_item[item_chunk(item_n)];
 
     __syncthreads();                                  // every wave is done with the previous tiles
 #pragma unroll
@@ -333,6 +374,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
         for (int i = 0; i < HW; ++i) lgp[WN - 1][i] = half2_t{ninf, ninf};   // stays if the row is left out
         fetch(KT{}, std::integral_constant<int, 0>{});
+        float held = 0.f;                               // raw sum of the even tap of a pair until its odd tap is done
         static_for<0, NSR>([&](auto s_tag) __attribute__((always_inline)) {
             constexpr int s = decltype(s_tag)::value, j = s / SPR, i0 = (s % SPR) * G;
             if constexpr (s + 1 < NSR) {
@@ -342,19 +384,43 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
             for (int t = 0; t < G; ++t) {
                 const int i = i0 + t;
-                float sum = l1_sum<T>(qv[0], buf[s & 1][t][0]);
+                float sum;
+                if constexpr (kMatrixSum) {
+                    f32x4_t acc4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int u = 1; u < VPL; ++u) sum += l1_sum<T>(qv[u], buf[s & 1][t][u]);   // per vector, then added: the
-                                                  // same bits whichever order the lane holds its vectors in
-                sum = group_sum<LPH>(sum);
-                const half_t l16 = (half_t)sum;                       // channel sum stored in fp16
-                const half_t s16 = (half_t)((float)l16 * nscale);     // scaled logit stored in fp16
-                if (i & 1) lgp[j][i >> 1].y = s16; else lgp[j][i >> 1].x = s16;
-                // pin the finished logit here: left alone, the optimiser gathers the last add and the
-                // conversions of all taps at the end of the phase and keeps every partial sum alive
-                uint32_t pinned = h2_as_u32(lgp[j][i >> 1]);
-                asm volatile("" : "+v"(pinned));
-                lgp[j][i >> 1] = as_h2(pinned);
+                    for (int u = 0; u < VPL; ++u) {
+                        u32x4 ad;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            ad[e] = h2_as_u32(as_h2(qv[u][e]) - as_h2(buf[s & 1][t][u][e])) & 0x7fff7fffu;
+                        acc4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(pair_ones, __builtin_bit_cast(half8_t, ad), acc4, 0, 0, 0);
+                    }
+                    sum = acc4[0];
+                } else {
+                    sum = l1_sum<T>(qv[0], buf[s & 1][t][0]);
+#pragma unroll
+                    for (int u = 1; u < VPL; ++u) sum += l1_sum<T>(qv[u], buf[s & 1][t][u]);   // per vector, then added: the
+                                                      // same bits whichever order the lane holds its vectors in
+                    sum = group_sum<LPH>(sum);
+                }
+                // the two roundings of a logit (channel sum to fp16, scaled logit to fp16) on a pair of taps at a
+                // time: two packed conversions and two multiplications for what took four instructions per tap
+                if (!(i & 1)) {
+                    held = sum;
+                    asm volatile("" : "+v"(held));
+                } else {
+                    typedef float float2_t __attribute__((ext_vector_type(2)));
+                    const half2_t l16 = __builtin_convertvector(float2_t{held, sum}, half2_t);
+                    // (float)half * scale in one instruction per half (the compiler's own choice is a conversion and a
+                    // multiplication each)
+                    float f_lo, f_hi;
+                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(f_lo) : "v"(h2_as_u32(l16)), "v"(nscale));
+                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(f_hi) : "v"(h2_as_u32(l16)), "v"(nscale));
+                    lgp[j][i >> 1] = __builtin_convertvector(float2_t{f_lo, f_hi}, half2_t);
+                    uint32_t pinned = h2_as_u32(lgp[j][i >> 1]);
+                    asm volatile("" : "+v"(pinned));
+                    lgp[j][i >> 1] = as_h2(pinned);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -460,10 +526,31 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
         for (int u = 0; u < VPL; ++u)
             buf_store16(ro, mine ? (uint32_t)pix * A.out_row_bytes + chan_bytes + vec_off[u] : kDeadOffset, ov[u]);
-        const uint32_t a_off = (mine && sub == 0) ? (uint32_t)pix * A.attn_row_bytes + (uint32_t)head * (uint32_t)(M * 2) : kDeadOffset;
+        // The attention row of a head-query (M/2 dwords) leaves in 16-byte pieces dealt to the LPH lanes of the
+        // head-query -- piece p from lane p % LPH -- so that one store instruction covers LPH * 16 contiguous bytes per
+        // head-query (8-byte stores from one lane made nine requests to L2 per row, three quarters of all the
+        // requests of the kernel).  The dwords left over (2 at M = 36) follow as one 8-byte store.
+        {
+            constexpr int NDW = M / 2, NP = NDW / 4, REM = NDW - NP * 4;
+            uint32_t dw[NDW];
 #pragma unroll
-        for (int m = 0; m < M / 2; m += 2)   // dword m of the row holds taps 2m, 2m+1
-            buf_store8(ra, a_off + m * 4, u32x2{h2_as_u32(ap[m / HW][m % HW]), h2_as_u32(ap[(m + 1) / HW][(m + 1) % HW])});
+            for (int m = 0; m < NDW; ++m) dw[m] = h2_as_u32(ap[m / HW][m % HW]);
+            const uint32_t a_row = mine ? (uint32_t)pix * A.attn_row_bytes + (uint32_t)head * (uint32_t)(M * 2) : kDeadOffset;
+#pragma unroll
+            for (int t = 0; t * LPH < NP; ++t) {
+                u32x4 piece = u32x4{dw[0], dw[1], dw[2], dw[3]};
+#pragma unroll
+                for (int sl = 0; sl < LPH; ++sl) {
+                    const int pc = t * LPH + sl;
+                    if (pc < NP && sub == sl) piece = u32x4{dw[4 * pc], dw[4 * pc + 1], dw[4 * pc + 2], dw[4 * pc + 3]};
+                }
+                const int mine_pc = t * LPH + sub;
+                buf_store16(ra, (mine && mine_pc < NP) ? a_row + (uint32_t)mine_pc * 16u : kDeadOffset, piece);
+            }
+            static_assert(REM == 0 || REM == 2, "attention rows are a whole number of 8-byte pieces");
+            if (REM == 2)
+                buf_store8(ra, (mine && sub == NP % LPH) ? a_row + (uint32_t)NP * 16u : kDeadOffset, u32x2{dw[NP * 4], dw[NP * 4 + 1]});
+        }
 
         slot += QPP;
         pix = pix_n; pix_n = pix_nn; xyu = xyu_n;
