@@ -580,7 +580,9 @@ int matchattn_forward_fused(const void *position, int position_heads, const void
 }
 
 namespace {
-struct BwdLayout { size_t sort_off, centre_off, dl_off, a_off, tile_off, total; SortLayout sl; bool tile; TileLayout tl; };
+struct BwdLayout { size_t sort_off, centre_off, dl_off, tile_off, total; SortLayout sl; bool tile; TileLayout tl; };
+// bytes of one (logit gradient, attention value) pair: two floats for fp32 tensors, two halves otherwise (PairOf<T>)
+size_t pair_bytes(int dtype) { return dtype == MATCHATTN_F32 ? 8 : 4; }
 // Whether pass A of the gather backward would run on LDS tiles (shapes the tile kernels have; the (dl, a)
 // scratch must fit the 32-bit offsets of a buffer descriptor).
 bool bwd_tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
@@ -589,7 +591,7 @@ bool bwd_tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx
     const int head_bytes = CH * (int)elem_size(dtype);
     if (!(rx <= 2 && (CH == 16 || CH == 32 || (CH == 64 && dtype != MATCHATTN_F32)) &&
           h % (head_bytes >= 128 ? 1 : 128 / head_bytes) == 0 &&
-          (unsigned long long)B * H * W * h * M * 8 < 0xFFFFF000ull))
+          (unsigned long long)B * H * W * h * M * pair_bytes(dtype) < 0xFFFFF000ull))
         return false;
     return mode == 1 || (long long)B * H * W * h >= (1ll << 18);   // auto: maps large enough to pay for the bucketing
 }
@@ -601,8 +603,7 @@ BwdLayout bwd_gather_layout(const Options &O, int B, int H, int W, int C, int h,
     l.sort_off = 0;
     l.centre_off = up(l.sl.total);
     l.dl_off = l.centre_off + up((size_t)B * H * W * h * 4);
-    l.a_off = l.dl_off + up(nhq * M * 4);
-    l.tile_off = l.a_off + up(nhq * M * 4);
+    l.tile_off = l.dl_off + up(nhq * M * pair_bytes(dtype));
     l.total = l.tile_off;
     l.tile = bwd_tile_wanted(O, B, H, W, C, h, rx, dtype);
     if (l.tile) {
@@ -665,7 +666,7 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
     ma::BwdArgs A;
     A.mo = max_offset; A.q = q; A.k = k; A.v = v; A.d_out = d_out; A.d_attn = d_attn;
     A.dq = dq; A.dmo = d_max_offset;
-    A.dl_ws = nullptr; A.a_ws = nullptr; A.dk = dk; A.dv = dv;
+    A.dl_ws = nullptr; A.dk = dk; A.dv = dv;
     A.perm = nullptr; A.centre = nullptr; A.bin_start = nullptr; A.row_start = nullptr; A.per_head = nullptr; A.nrows = B * H;
     A.only_flagged = nullptr;
     A.nhq = (int)(L * h); A.N = H * W; A.H = H; A.W = W; A.C = C; A.h = h;
@@ -687,7 +688,7 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
             launch_sort(S, sl, L, h, ws, true, s);
             if (hipError_t e = hipGetLastError())
                 return fail(MATCHATTN_ERR_LAUNCH, "matchattn_backward: index launch failed: %s", hipGetErrorString(e));
-            A.dl_ws = (float *)(ws + bl.dl_off); A.a_ws = A.dl_ws + 1;      // interleaved (dl, a) pairs
+            A.dl_ws = ws + bl.dl_off;                                       // (dl, a) pairs
             A.dk_acc = nullptr; A.dv_acc = nullptr;
             A.perm = S.perm; A.centre = S.centre; A.bin_start = S.count; A.row_start = S.rowtot; A.per_head = S.per_head;
             const char *kname = "";

@@ -21,8 +21,8 @@ struct BwdArgs {
     float *dk_acc, *dv_acc;                       // scatter mode: fp32 [B*N*C], zero on entry
     // gather mode (deterministic, no atomics): pass A leaves, per head-query and tap, the logit
     // gradient and the attention weight; pass B sums them per key through the inverse index
-    float *dl_ws, *a_ws;                          // one array [B*N*h][M][2] = (dl, a) pairs (a_ws = dl_ws + 1: pass B
-                                                  //   fetches both with one 8-byte load), or null in scatter mode
+    void *dl_ws;                                  // one array [B*N*h][M] of (dl, a) pairs (PairOf<T>: pass B fetches both
+                                                  //   with one load), or null in scatter mode
     void *dk, *dv;                                // outputs of pass B (dtype T)
     const int *perm, *centre, *bin_start, *row_start, *per_head;   // inverse index (matchattn_sort.h), exact bins
     const uint8_t *only_flagged;                  // pass A: optional [nhq] flags, compute only the head-queries whose flag is set
@@ -31,6 +31,30 @@ struct BwdArgs {
     int N, H, W, C, h;
     float scale;
     int xcd_swizzle;
+};
+
+// The (logit gradient, attention value) pair pass A leaves per head-query and tap for pass B.  fp32 tensors keep two
+// floats; 16-bit tensors keep two halves in one word: the attention value is a 16-bit number by definition, and the
+// logit gradient, rounded to half precision (11 bits, like every gradient the call returns; saturated at the largest
+// half instead of overflowing), halves what pass A writes and pass B reads through L2 per tap.
+template <typename T> struct PairOf {
+    static constexpr int kBytes = 4;
+    typedef uint32_t Word;
+    static __device__ __forceinline__ Word pack(float dl, float a) {
+        const float s = __builtin_amdgcn_fmed3f(dl, -65504.0f, 65504.0f);
+        return h2_as_u32(half2_t{(half_t)s, (half_t)a});
+    }
+    static __device__ __forceinline__ void unpack(Word w, float &dl, float &a) {
+        const half2_t h = as_h2(w);
+        dl = (float)h.x;
+        a = (float)h.y;
+    }
+};
+template <> struct PairOf<float> {
+    static constexpr int kBytes = 8;
+    typedef u32x2 Word;
+    static __device__ __forceinline__ Word pack(float dl, float a) { return u32x2{as_u32(dl), as_u32(a)}; }
+    static __device__ __forceinline__ void unpack(Word w, float &dl, float &a) { dl = as_f32(w[0]); a = as_f32(w[1]); }
 };
 
 __device__ __forceinline__ void atomic_add_f32(float *p, float v) { unsafeAtomicAdd(p, v); }
@@ -221,12 +245,12 @@ __global__ __launch_bounds__(256, R == 1 ? 3 : (GATHER ? MA_BWD_WAVES_R2 : 1)) v
         dm[0] = Tr::from_f(dx);
         dm[1] = Tr::from_f(dy);
         if constexpr (GATHER) {
-            float2 *dst = (float2 *)A.dl_ws + (size_t)hq * M;
+            typename PairOf<T>::Word *dst = (typename PairOf<T>::Word *)A.dl_ws + (size_t)hq * M;
 #pragma unroll
             for (int j = 0; j < WN; ++j)
 #pragma unroll
                 for (int i = 0; i < WN; ++i)
-                    dst[j * WN + i] = float2{g[j][i], Tr::round(attn_value<R>(shared, lg, st, c9, j, i))};
+                    dst[j * WN + i] = PairOf<T>::pack(g[j][i], Tr::round(attn_value<R>(shared, lg, st, c9, j, i)));
         }
     }
 

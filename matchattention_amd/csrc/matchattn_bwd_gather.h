@@ -187,17 +187,21 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
                 const int i_lo = info & 7, i_hi = (info >> 3) & 7, j_lo = (info >> 6) & 7, j_hi = (info >> 9) & 7;
                 const int qhq = qp * A.h + head;
                 if constexpr (ONE) {
-                    const float2 da = *(const float2 *)(A.dl_ws + ((size_t)qhq * M + (hit ? j_lo * WN + i_lo : 0)) * 2);
-                    bt.dl[u] = hit ? da.x : 0.f;
-                    bt.am[u] = hit ? da.y : 0.f;
+                    const typename PairOf<T>::Word da = ((const typename PairOf<T>::Word *)A.dl_ws)[(size_t)qhq * M + (hit ? j_lo * WN + i_lo : 0)];
+                    float dl_t, a_t;
+                    PairOf<T>::unpack(da, dl_t, a_t);
+                    bt.dl[u] = hit ? dl_t : 0.f;
+                    bt.am[u] = hit ? a_t : 0.f;
                 } else {
                     bt.dl[u] = 0.f; bt.am[u] = 0.f;
                     if (hit) {                          // several taps of one query on this key simply add up
                         for (int j = j_lo; j <= j_hi; ++j)
                             for (int i = i_lo; i <= i_hi; ++i) {
-                                const float2 da = *(const float2 *)(A.dl_ws + ((size_t)qhq * M + j * WN + i) * 2);
-                                bt.dl[u] += da.x;
-                                bt.am[u] += da.y;
+                                const typename PairOf<T>::Word da = ((const typename PairOf<T>::Word *)A.dl_ws)[(size_t)qhq * M + j * WN + i];
+                                float dl_t, a_t;
+                                PairOf<T>::unpack(da, dl_t, a_t);
+                                bt.dl[u] += dl_t;
+                                bt.am[u] += a_t;
                             }
                     }
                 }

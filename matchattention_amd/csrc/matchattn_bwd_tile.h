@@ -39,7 +39,7 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
     const __amdgpu_buffer_rsrc_t rm = make_rsrc(A.mo, (uint32_t)A.nhq * 4u);
     const __amdgpu_buffer_rsrc_t rdm = make_rsrc(A.dmo, (uint32_t)A.nhq * 4u);
     const __amdgpu_buffer_rsrc_t rda = make_rsrc(A.d_attn, A.d_attn ? (uint32_t)A.nhq * (uint32_t)(M * 2) : 0u);
-    const __amdgpu_buffer_rsrc_t rws = make_rsrc(A.dl_ws, (uint32_t)A.nhq * (uint32_t)(M * 8));
+    const __amdgpu_buffer_rsrc_t rws = make_rsrc(A.dl_ws, (uint32_t)A.nhq * (uint32_t)(M * 4));   // (dl, a) as two halves per tap
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(S.defer, (uint32_t)A.nhq);
     const int sub = threadIdx.x % LPH;
     const int grp = threadIdx.x / LPH;
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
             const bool mine = valid && fits && !far;
             // (the dead offset leaves room for the tap offsets added below: kDeadOffset + 280 would wrap to a valid one;
             // the host keeps the scratch array below 0xFFFFF000 bytes)
-            const uint32_t ws_off = (mine && sub == 0) ? (uint32_t)hq * (uint32_t)(M * 8) : 0xFFFFF000u;
+            const uint32_t ws_off = (mine && sub == 0) ? (uint32_t)hq * (uint32_t)(M * 4) : 0xFFFFF000u;
 #pragma unroll
             for (int j = 0; j < WN; ++j)
 #pragma unroll
@@ -320,9 +320,9 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
                         a2[d] = (float)(half_t)(e[j][i + d] * cc);                // the stored attention value
                         g[j][i + d] = dl2[d];
                     }
-                    // (dl, a) pairs of two taps: one 16-byte store
-                    __builtin_amdgcn_raw_buffer_store_b128(u32x4{as_u32(dl2[0]), as_u32(a2[0]), as_u32(dl2[1]), as_u32(a2[1])}, rws,
-                                                           (int)(ws_off + (uint32_t)((j * WN + i) * 8)), 0, 0);
+                    // (dl, a) pairs of two taps: one 8-byte store
+                    buf_store8(rws, ws_off + (uint32_t)((j * WN + i) * 4),
+                               u32x2{PairOf<T>::pack(dl2[0], a2[0]), PairOf<T>::pack(dl2[1], a2[1])});
                 }
             {
                 float dx, dy;

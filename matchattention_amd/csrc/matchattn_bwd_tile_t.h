@@ -33,7 +33,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArg
     const __amdgpu_buffer_rsrc_t rm = make_rsrc(A.mo, (uint32_t)A.nhq * (uint32_t)(2 * ES));
     const __amdgpu_buffer_rsrc_t rdm = make_rsrc(A.dmo, (uint32_t)A.nhq * (uint32_t)(2 * ES));
     const __amdgpu_buffer_rsrc_t rda = make_rsrc(A.d_attn, A.d_attn ? (uint32_t)A.nhq * (uint32_t)(M * ES) : 0u);
-    const __amdgpu_buffer_rsrc_t rws = make_rsrc(A.dl_ws, (uint32_t)A.nhq * (uint32_t)(M * 8));
+    const __amdgpu_buffer_rsrc_t rws = make_rsrc(A.dl_ws, (uint32_t)A.nhq * (uint32_t)(M * PairOf<T>::kBytes));
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(S.defer, (uint32_t)A.nhq);
     const int sub = threadIdx.x % LPH;
     const int grp = threadIdx.x / LPH;
@@ -230,13 +230,16 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArg
                 }
                 // (a dead offset with room for the whole row: M * 8 bytes added to kDeadOffset would wrap into the
                 // array; the host keeps the array below 0xFFFFF000 bytes)
-                const uint32_t p_off = wr ? (uint32_t)hq * (uint32_t)(M * 8) : 0xFFFFF000u;
+                const uint32_t p_off = wr ? (uint32_t)hq * (uint32_t)(M * PairOf<T>::kBytes) : 0xFFFFF000u;
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
 #pragma unroll
                     for (int i = 0; i < WN; ++i)
-                        buf_store8(rws, p_off + (uint32_t)((j * WN + i) * 8),
-                                   u32x2{as_u32(g[j][i]), as_u32(Tr::round(attn_value<R>(shared, lg, st, c9, j, i)))});
+                    {
+                        const auto pw = PairOf<T>::pack(g[j][i], Tr::round(attn_value<R>(shared, lg, st, c9, j, i)));
+                        if constexpr (PairOf<T>::kBytes == 8) buf_store8(rws, p_off + (uint32_t)((j * WN + i) * 8), pw);
+                        else __builtin_amdgcn_raw_buffer_store_b32(pw, rws, (int)(p_off + (uint32_t)((j * WN + i) * 4)), 0, 0);
+                    }
             }
 
             // ---- dQ = -sum_m dl_m sgn(q - k_m) -----------------------------------------------------------

@@ -32,8 +32,9 @@ def test_host_only_entry_points_work_without_a_gpu():
     # head size without a tiled kernel: atomic mode only (fp32 accumulates in place; 16-bit types stage in fp32)
     assert lib.matchattn_backward_workspace_bytes(1, 8, 8, 48, 4, 1, 1, _cabi.F32) == 0
     assert lib.matchattn_backward_workspace_bytes(1, 8, 8, 48, 4, 1, 1, _cabi.F16) == 2 * 8 * 8 * 48 * 4
-    # tiled shapes: per-tap scratch (2 x nhq x M fp32) and the inverse index on top
-    assert lib.matchattn_backward_workspace_bytes(1, 8, 8, 32, 4, 1, 1, _cabi.F16) > 2 * 8 * 8 * 4 * 16 * 4
+    # tiled shapes: per-tap scratch (nhq x M pairs: two floats in fp32, two halves otherwise) and the inverse index on top
+    assert lib.matchattn_backward_workspace_bytes(1, 8, 8, 32, 4, 1, 1, _cabi.F16) > 8 * 8 * 4 * 16 * 4
+    assert lib.matchattn_backward_workspace_bytes(1, 8, 8, 32, 4, 1, 1, _cabi.F32) > 8 * 8 * 4 * 16 * 8
     assert lib.matchattn_set_option(b"no_such_option", 1) == 1
     assert b"unknown option" in lib.matchattn_last_error()
     assert lib.matchattn_set_option(b"forward_variant", 3) == 1
