@@ -203,6 +203,40 @@ def _e2e_ms_per_frame(only_size=None):
     return out
 
 
+def _e2e_pytorch_baseline():
+    """The baseline legs of the end-to-end plan: the same harness with the operator in plain PyTorch ops
+    (`mat_impl='pytorch'`, matchattention_amd.mat_torch) at 1280x720 -- on the GPU in fp16 with the 5 + 5 protocol, and
+    on the host cores in fp32, one frame."""
+    import torch
+    from matchattention_amd.mat_torch import attend_torch
+    from matchattention_amd.stereo_harness import MatchStereoHarness
+    from matchattention_amd.workloads import make_stereo_pair
+    out = {}
+    model = MatchStereoHarness(attend_torch, "tiny", seed=0).cuda().half().eval()
+    left, right, _ = make_stereo_pair(720, 1280, dtype=torch.float16)
+    with torch.inference_mode():
+        for _ in range(5):
+            model(left, right)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            model(left, right)
+        b.record()
+        torch.cuda.synchronize()
+    out["1280x720_ms_per_frame_pytorch_operator_gpu_fp16"] = round(a.elapsed_time(b) / 5, 3)
+    del model
+    torch.cuda.empty_cache()
+    model = MatchStereoHarness(attend_torch, "tiny", seed=0).eval()
+    left, right, _ = make_stereo_pair(720, 1280, device="cpu", dtype=torch.float32)
+    with torch.inference_mode():
+        t0 = time.perf_counter()
+        model(left, right)
+        out["1280x720_ms_per_frame_pytorch_operator_cpu_fp32"] = round((time.perf_counter() - t0) * 1e3, 1)
+    out["cpu_threads"] = _cpu_threads()
+    return out
+
+
 def _module_step_ms(wl, inp, steps=20):
     """The cross-attention module's sequence around the operator at this workload's size -- pixel grid add,
     clamp, operator, gate, concatenation (reference models/attention_blocks.py:162-163, 45-59, 96-98) -- as
@@ -443,6 +477,8 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
         extra["e2e_matchstereo_tiny"] = _e2e_ms_per_frame()
+        if not args.no_cpu:
+            extra["e2e_matchstereo_tiny"].update(_e2e_pytorch_baseline())
 
     cpu = None
     if not args.no_cpu:

@@ -110,7 +110,8 @@ int matchattn_forward_static(const void *max_offset, const void *q, const void *
  *
  * The workspace (matchattn_forward_fused_workspace_bytes, 16-byte aligned) is required when
  * position_heads != 0; it receives the sampling positions and serves the kernels as in matchattn_forward_ws.
- * Inference only: matchattn_backward differentiates the unfused operator.
+ * matchattn_backward differentiates the operator itself; a binding that trains through this call applies the gate's
+ * and the clamp's own gradients around it (matchattention_amd/match_former_ops.py does).
  */
 size_t matchattn_forward_fused_workspace_bytes(int B, int H, int W, int C, int h, int rx, int ry, int dtype);
 int matchattn_forward_fused(const void *position, int position_heads,

@@ -233,19 +233,77 @@ def _(position, q, k, v, gate, H, W, win_r, num_head, scale, relative, concat):
     return torch.empty_like(q), q.new_empty((B, N, num_head, M))
 
 
+def _sampling_positions(position: torch.Tensor, H: int, W: int, r: int, h: int, relative: bool):
+    """What the fused call computes before the operator, in torch ops: pixel grid add and clamp with the bounds
+    rounded to the tensor dtype (models/attention_blocks.py:149-151, 162-163, 45-59).  Returns the sampling
+    positions [B,N,h,2] and the mask of the components the clamp let through (its gradient)."""
+    B, N = position.shape[:2]
+    if not relative:
+        return position, None
+    dt, dev = position.dtype, position.device
+    ys, xs = torch.meshgrid(torch.arange(H, device=dev, dtype=dt), torch.arange(W, device=dev, dtype=dt), indexing="ij")
+    grid = torch.stack((xs, ys), -1).view(1, N, 1, 2)
+    raw = (position + grid).expand(B, N, h, 2)
+    lo = torch.full((), float(r), dtype=dt, device=dev)
+    hi = torch.stack((torch.full((), W - 1 - r - 1e-3, dtype=dt, device=dev), torch.full((), H - 1 - r - 1e-3, dtype=dt, device=dev)))
+    mo = torch.minimum(torch.maximum(raw, lo), hi)
+    return mo.contiguous(), (raw >= lo) & (raw <= hi)
+
+
+def _fused_setup_context(ctx, inputs, output):
+    position, q, k, v, gate, H, W, win_r, num_head, scale, relative, concat = inputs
+    ctx.save_for_backward(position, q, k, v, gate)
+    ctx.cfg = (H, W, list(win_r), int(num_head), float(scale), bool(relative), bool(concat))
+
+
+def _fused_backward(ctx, d_first, d_second):
+    """Gradient of the fused module step: the column ranges of the projection input are split back into the
+    gradient of the gated output and of the attention weights, the gate takes d(gate * out) -- `out` is recomputed
+    by one forward call, the fused forward stores only the product --, the operator's backward kernel does the
+    rest, and the clamp's mask and the broadcast over heads turn d max_offset into d position."""
+    position, q, k, v, gate = ctx.saved_tensors
+    H, W, win_r, h, scale, relative, concat = ctx.cfg
+    B, N, C = q.shape
+    M = (2 * win_r[0] + 2) * (2 * win_r[1] + 2)
+    mo, passed = _sampling_positions(position, H, W, win_r[0], h, relative)
+    if concat:
+        d_res = None if d_first is None else d_first[..., :C]
+        d_attn = None if d_first is None else d_first[..., C:].reshape(B, N, h, M).contiguous()
+    else:
+        d_res, d_attn = d_first, d_second
+    if d_res is None:
+        d_res = torch.zeros_like(q)
+    d_gate = None
+    if gate is not None:
+        out = torch.empty_like(q)
+        attn = q.new_empty((B, N, h, M))
+        fused_forward_ops(mo, q, k, v, out, attn, H, W, win_r, M, "l1_norm", scale)
+        d_gate = d_res * out
+        d_res = d_res * gate
+    dq, dk, dv, dmo = match_attention_backward(mo, q, k, v, d_res.contiguous(), d_attn, H, W, win_r, scale)
+    if relative:
+        dmo = dmo * passed
+        if position.size(2) == 1 and h > 1:
+            dmo = dmo.sum(2, keepdim=True)
+    return dmo, dq, dk, dv, d_gate, None, None, None, None, None, None, None
+
+
+fused_module_step.register_autograd(_fused_backward, setup_context=_fused_setup_context)
+
+
 def fused_module_forward(position: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                          H: int, W: int, win_r: List[int], num_head: int, scale: float,
                          gate: Optional[torch.Tensor] = None, relative: bool = True, concat: bool = False):
     """The operator together with the elementwise steps the attention module runs either side of it, in
-    one native call (inference only; ``matchattn_forward_fused`` of the C ABI).
+    one native call (``matchattn_forward_fused`` of the C ABI); differentiable.
 
     ``position`` [B,N,hp,2]: with ``relative`` the positions relative to each query pixel, hp = num_head or
     1 (shared by all heads) -- the pixel coordinates are added and the sum clamped inside the call, as
     models/attention_blocks.py:149-151 / 162-163 and :45-59 do; otherwise the clamped sampling positions
     (hp = num_head).  ``gate`` [B,N,C] multiplies the output (:96).  With ``concat`` the result is the single
-    [B,N,C + h*attn_num] tensor the cross-attention projection consumes (:97-98); otherwise (out, attn)."""
-    if torch.is_grad_enabled() and any(t.requires_grad for t in (position, q, k, v) + ((gate,) if gate is not None else ())):
-        raise RuntimeError("fused_module_forward is inference-only; use MF_FusedForwardOps for training")
+    [B,N,C + h*attn_num] tensor the cross-attention projection consumes (:97-98); otherwise (out, attn).
+    Under autograd the backward recomputes the ungated output with one forward call and runs the operator's
+    backward kernel; gradients flow to position (through the clamp's mask), q, k, v and gate."""
     first, second = fused_module_step(position, q, k, v, gate, H, W, list(win_r), int(num_head), float(scale),
                                       bool(relative), bool(concat))
     return first if concat else (first, second)

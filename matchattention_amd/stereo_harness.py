@@ -12,8 +12,7 @@ The operator is injected: ``attend(max_offset, q, k, v, H, W, win_r, attn_num, s
 choice; tests plug a PyTorch definition for the 'pytorch' one.  Optionally a second callable,
 ``fused(position, q, k, v, H, W, win_r, num_head, scale, gate=, relative=True, concat=)``
 (``matchattention_amd.fused_module_forward``), takes over the elementwise steps either side of the
-operator when no gradient is needed: the pixel-coordinate add and clamp before it, the gate and the
-concatenation after it.
+operator: the pixel-coordinate add and clamp before it, the gate and the concatenation after it.
 """
 import math
 from typing import Callable, List, Optional, Sequence
@@ -198,18 +197,20 @@ class MatchAttention(nn.Module):
         else:
             ref = tgt = torch.cat((x, noc_mask.reshape(B, N, 1)), -1)
         q, k, v = self.q(ref).contiguous(), self.k(tgt).contiguous(), self.v(tgt).contiguous()
-        if self.fused is not None and not (torch.is_grad_enabled() and (x.requires_grad or rel.requires_grad)):
+        if self.fused is not None:
             res = self.fused(rel.contiguous(), q, k, v, H, W, [r, r], self.h, self.scale,
                              gate=gate.contiguous() if self.cross else None, relative=True, concat=self.cross)
             return self.proj(res if self.cross else res[0]).view(B, H, W, -1)
         max_offset = (rel + pixel_grid(B, H, W, rel.dtype, rel.device).reshape(B, N, 1, 2)).expand(B, N, self.h, 2)
-        # clamp with the bounds rounded to the tensor dtype as the reference does (:45-59); the rounding
-        # is done on the host so that the forward stays capturable in a HIP graph (no host-to-device copy)
-        dt = max_offset.dtype
-        hi_x = float(torch.tensor(W - 1 - r - 1e-3, dtype=dt))
-        hi_y = float(torch.tensor(H - 1 - r - 1e-3, dtype=dt))
-        mx = torch.clamp(max_offset[..., 0:1], min=float(r), max=hi_x)
-        my = torch.clamp(max_offset[..., 1:2], min=float(r), max=hi_y)
+        # clamp with the bounds rounded to the tensor dtype as the reference does (:45-59); the bounds are filled on
+        # the device (no host-to-device copy, no host read-back: the forward stays capturable in a HIP graph and
+        # traces under torch.compile without a graph break)
+        dt, dev = max_offset.dtype, max_offset.device
+        lo = torch.full((), float(r), dtype=dt, device=dev)
+        hi_x = torch.full((), W - 1 - r - 1e-3, dtype=dt, device=dev)
+        hi_y = torch.full((), H - 1 - r - 1e-3, dtype=dt, device=dev)
+        mx = torch.clamp(max_offset[..., 0:1], min=lo, max=hi_x)
+        my = torch.clamp(max_offset[..., 1:2], min=lo, max=hi_y)
         out, attn = self.attend(torch.cat((mx, my), -1).contiguous(), q, k, v, H, W, [r, r], self.M, self.scale)
         if self.cross:
             out = torch.cat((gate * out, attn.reshape(B, N, -1)), -1)
@@ -307,16 +308,18 @@ class MatchStereoHarness(nn.Module):
                     if m.bias is not None:
                         m.bias.zero_()
 
-    def forward(self, left, right):
+    def forward(self, left, right, init_field=None, return_rpos=False):
         """left, right: [B,3,H,W] in 0..255, H and W multiples of 32.  Returns the full-resolution
         field [2B,H,W,2] (x-disparity of the left view in the first half, of the right view in the
-        second) and the list of per-scale fields."""
+        second) and the list of per-scale fields; with `return_rpos` also the self-attention's relative
+        positions at 1/4 scale [2B,H/4,W/4,2].  `init_field` [2B,H/32,W/32,2] replaces the initial
+        correlation (the low-resolution initialisation of the reference's script, match_stereo.py:96-103)."""
         x = torch.cat((2 * (left / 255.0) - 1, 2 * (right / 255.0) - 1), 0).contiguous()
         feats = self.encoder(x)[::-1]
         fields = []
         for i in range(4):
             if i == 0:
-                field = self.init_corr(feats[0])
+                field = self.init_corr(feats[0]) if init_field is None else init_field.to(feats[0].dtype).clone()
                 rpos = torch.zeros_like(field)
             else:
                 feats[i] = self.fuse[i - 1](feats[i - 1], feats[i])
@@ -332,4 +335,6 @@ class MatchStereoHarness(nn.Module):
             rpos = rp.view(B2, H, W, h, 2).mean(-2)
             fields.append(field)
         full = convex_upsample(field, self.final_mask(feats[-1].permute(0, 3, 1, 2)), 4)
+        if return_rpos:
+            return full, fields, rpos
         return full, fields

@@ -84,5 +84,3 @@ def test_fused_entry_validates_before_any_gpu_call():
         fused_module_forward(torch.zeros(1, 64, 3, 2), q, q, q, 8, 8, [1, 1], 4, 1.0)
     with pytest.raises(ValueError, match="GPU tensor"):
         fused_module_forward(torch.zeros(1, 64, 1, 2), q, q, q, 8, 8, [1, 1], 4, 1.0)
-    with pytest.raises(RuntimeError, match="inference-only"):
-        fused_module_forward(torch.zeros(1, 64, 1, 2), q.clone().requires_grad_(True), q, q, 8, 8, [1, 1], 4, 1.0)

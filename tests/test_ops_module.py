@@ -65,3 +65,52 @@ def test_fused_module_step_is_an_opaque_op_too(hip_lib):
         assert torch.library.opcheck(torch.ops.matchattention_amd.fused_module_step,
                                      (rel, q, k, v, gate if concat else None, H, W, [r, r], h, 0.25, True, concat),
                                      test_utils=("test_schema", "test_faketensor"))
+
+
+@pytest.mark.parametrize("dt,shared,gated,concat", [(torch.float32, True, True, True), (torch.float32, False, False, False),
+                                                    (torch.float16, True, True, True), (torch.float16, False, True, False)])
+def test_fused_module_step_trains_like_the_separate_steps(hip_lib, dt, shared, gated, concat):
+    # gradients of the one-call module step (grid add, clamp, operator, gate, concatenation) against autograd through
+    # the same steps written out in torch ops around the oracle, in fp64 on the same rounded inputs; some positions lie
+    # outside the clamp's range, so its mask matters
+    from matchattention_amd import fused_module_forward
+    from tests.util import TOL, check_err
+    B, H, W, h, Ch, r = 2, 12, 14, 4, 16, 2
+    N, C, M = H * W, h * Ch, 36
+    g = torch.Generator().manual_seed(21)
+    q, k, v = (torch.randn(B, N, C, generator=g).to(dt) for _ in range(3))
+    rel = (torch.randn(B, N, 1 if shared else h, 2, generator=g) * 4.0).to(dt)
+    gate = torch.rand(B, N, C, generator=g).to(dt) if gated else None
+    d_res = torch.randn(B, N, C + (h * M if concat else 0), generator=g).to(dt)
+    d_attn = None if concat else torch.randn(B, N, h, M, generator=g).to(dt)
+    scale = Ch ** -0.5
+
+    # reference: the separate steps in fp64
+    ins64 = [t.double().requires_grad_(True) for t in (rel, q, k, v)] + ([gate.double().requires_grad_(True)] if gated else [])
+    grid = O.init_coords(B, H, W, dtype=torch.float64).view(B, N, 1, 2)
+    raw = ins64[0] + grid
+    raw = (raw + (raw.detach().to(dt).double() - raw.detach())).expand(B, N, h, 2)   # the sum is stored in the tensor dtype
+    lo = float(r)
+    hx, hy = (float(torch.tensor(s - 1 - r - 1e-3, dtype=dt)) for s in (W, H))
+    mo = torch.cat((raw[..., 0:1].clamp(lo, hx), raw[..., 1:2].clamp(lo, hy)), -1)
+    out, attn = O.forward(mo, ins64[1], ins64[2], ins64[3], H, W, [r, r], scale)
+    if gated:
+        out = ins64[4] * out
+    if concat:
+        want = torch.autograd.grad([torch.cat((out, attn.reshape(B, N, -1)), -1)], ins64, [d_res.double()])
+    else:
+        want = torch.autograd.grad([out, attn], ins64, [d_res.double(), d_attn.double()])
+
+    dev = [t.cuda().requires_grad_(True) for t in (rel, q, k, v)] + ([gate.cuda().requires_grad_(True)] if gated else [])
+    res = fused_module_forward(dev[0], dev[1], dev[2], dev[3], H, W, [r, r], h, scale, gate=dev[4] if gated else None,
+                               relative=True, concat=concat)
+    if concat:
+        got = torch.autograd.grad([res], dev, [d_res.cuda()])
+    else:
+        got = torch.autograd.grad(list(res), dev, [d_res.cuda(), d_attn.cuda()])
+    clamped = float(((raw.detach()[..., 0] < lo) | (raw.detach()[..., 0] > hx)).float().mean())
+    assert clamped > 0.05                                   # the mask is exercised
+    tol = TOL[dt]
+    for a, b, name in zip(got, want, ("d_position", "dq", "dk", "dv", "d_gate")):
+        assert a.shape == b.shape and torch.isfinite(a).all(), name
+        check_err(a.cpu(), b, tol, f"fused step bwd {name} {str(dt).split('.')[1]}")
