@@ -108,8 +108,11 @@ int matchattn_forward_static(const void *max_offset, const void *q, const void *
  * pixel) every attn_row_stride elements (0: contiguous), so both can be column ranges of the [B,N,C+h*M]
  * input of the output projection: out = buf, attn = buf + C, both strides C + h*M.
  *
- * The workspace (matchattn_forward_fused_workspace_bytes, 16-byte aligned) is required when
- * position_heads != 0; it receives the sampling positions and serves the kernels as in matchattn_forward_ws.
+ * Workspace: matchattn_forward_fused_workspace_bytes returns what these sizes would use (16-byte aligned scratch), 0 for
+ * maps that do not take the LDS-tile path: there the kernel that runs adds the pixel grid and clamps in its own prologue
+ * and the call is a single launch.  On the LDS-tile path the sampling positions are first written to the head of the
+ * workspace by a pass of their own (the bucketing reads every position three times); a NULL workspace selects the
+ * single-launch kernels at any size.
  * matchattn_backward differentiates the operator itself; a binding that trains through this call applies the gate's
  * and the clamp's own gradients around it (matchattention_amd/match_former_ops.py does).
  */

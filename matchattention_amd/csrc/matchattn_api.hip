@@ -312,6 +312,9 @@ struct Placement {
     long long out_stride = 0, attn_stride = 0;
     const void *gate = nullptr;
     bool shared_offsets = false;    // every head of a pixel is known to have the same sampling position
+    // `max_offset` holds positions relative to the query pixels, [B,N,rel_heads,2] (0: the sampling positions
+    // themselves); set only for calls that take a kernel which adds the pixel grid and clamps in its own prologue
+    int rel_heads = 0;
 };
 
 int forward_impl(const Options &O, const void *max_offset, const void *q, const void *k, const void *v, void *out, void *attn,
@@ -338,6 +341,8 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
     A.scale = scale; A.row_skip = O.row_skip; A.xcd_swizzle = O.xcd_swizzle;
     A.defer = nullptr;
     A.out_row_bytes = (uint32_t)(out_stride * es); A.attn_row_bytes = (uint32_t)(attn_stride * es); A.gate = P.gate;
+    A.rel_heads = P.rel_heads;
+    A.lo_x = (float)rx; A.hi_x = (float)((double)(W - 1 - rx) - 1e-3); A.lo_y = (float)ry; A.hi_y = (float)((double)(H - 1 - ry) - 1e-3);
 
     const int variant = O.forward_variant;
     const char *kname = "";
@@ -348,7 +353,7 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
         const int vpl = variant > 0 ? variant : default_vpl(CH, rx, dtype);
         // LDS-tile path: bucket the queries by K/V tile, one workgroup per tile and head group, then the
         // generic kernel for the (normally empty) list of queries a tile could not serve
-        if (workspace && tile_wanted(O, B, H, W, C, h, rx, ry, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
+        if (workspace && P.rel_heads == 0 && tile_wanted(O, B, H, W, C, h, rx, ry, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
             const TileLayout tl = tile_layout(B, H, W, h);
             const SortLayout &sl = tl.sl;
             if (workspace_bytes < tl.total)
@@ -528,7 +533,10 @@ int matchattn_forward_deferred(const void *workspace, size_t workspace_bytes,
 
 size_t matchattn_forward_fused_workspace_bytes(int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
     if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || h <= 0) return 0;
-    return offsets_bytes(B, H, W, h, dtype) + forward_workspace_bytes(options_now(), B, H, W, C, h, rx, ry, dtype);
+    // only the LDS-tile path wants scratch: the sampling positions (a pass of their own prepares them for the bucketing,
+    // which reads every position three times) and the buckets; the other kernels take relative positions as they are
+    const size_t fw = forward_workspace_bytes(options_now(), B, H, W, C, h, rx, ry, dtype);
+    return fw ? offsets_bytes(B, H, W, h, dtype) + fw : 0;
 }
 
 int matchattn_forward_fused(const void *position, int position_heads, const void *q, const void *k, const void *v,
@@ -549,11 +557,20 @@ int matchattn_forward_fused(const void *position, int position_heads, const void
     P.shared_offsets = position_heads == 1;
     if (position_heads == 0)
         return forward_impl(O, position, q, k, v, out, attn, P, workspace, workspace_bytes, B, H, W, C, h, rx, ry, scale, dtype, stream);
-    // relative positions: the sampling positions go to the head of the workspace, the rest serves the kernels
+    // Relative positions.  Without the LDS-tile path (small maps, or no workspace) the kernel that runs adds the pixel grid
+    // and clamps in its own prologue: no launch beside it.  (Element-aligned positions are all that path needs.)
     const size_t ob = offsets_bytes(B, H, W, h, dtype);
-    if (!workspace || workspace_bytes < ob || (reinterpret_cast<uintptr_t>(workspace) & 15u))
+    const size_t fw = forward_workspace_bytes(O, B, H, W, C, h, rx, ry, dtype);
+    if (!fw || !workspace) {
+        if (reinterpret_cast<uintptr_t>(position) & (elem_size(dtype) - 1))
+            return fail(MATCHATTN_ERR_ARG, "matchattn_forward_fused: position is not aligned to its element size");
+        P.rel_heads = position_heads;
+        return forward_impl(O, position, q, k, v, out, attn, P, nullptr, 0, B, H, W, C, h, rx, ry, scale, dtype, stream);
+    }
+    // LDS-tile path: the sampling positions go to the head of the workspace, the rest serves the kernels
+    if (workspace_bytes < ob + fw || (reinterpret_cast<uintptr_t>(workspace) & 15u))
         return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_fused: a 16-byte aligned workspace of %zu bytes is needed, %zu given",
-                    ob + forward_workspace_bytes(O, B, H, W, C, h, rx, ry, dtype), workspace ? workspace_bytes : (size_t)0);
+                    ob + fw, workspace_bytes);
     const int nhq = B * H * W * h;
     const float lo_x = (float)rx, hi_x = (float)((double)(W - 1 - rx) - 1e-3), lo_y = (float)ry, hi_y = (float)((double)(H - 1 - ry) - 1e-3);
     const dim3 grid((unsigned)((nhq + 255) / 256)), block(256);
@@ -575,7 +592,7 @@ int matchattn_forward_fused(const void *position, int position_heads, const void
     if (hipError_t e = hipGetLastError())
         return fail(MATCHATTN_ERR_LAUNCH, "matchattn_forward_fused: launch failed: %s", hipGetErrorString(e));
     const size_t rest = workspace_bytes - ob;
-    return forward_impl(O, workspace, q, k, v, out, attn, P, rest ? (char *)workspace + ob : nullptr, rest, B, H, W, C, h, rx, ry, scale,
+    return forward_impl(O, workspace, q, k, v, out, attn, P, (char *)workspace + ob, rest, B, H, W, C, h, rx, ry, scale,
                         dtype, stream);
 }
 

@@ -28,6 +28,13 @@ struct FwdArgs {
     // (models/attention_blocks.py:96).
     uint32_t out_row_bytes, attn_row_bytes;
     const void *gate;
+    // Sampling positions.  rel_heads == 0: `mo` holds them, [pixels][h][2], already clamped by the caller.  Otherwise
+    // `mo` holds positions relative to each query pixel, [pixels][rel_heads][2] with rel_heads == h, or 1 for one
+    // position every head shares, and the kernel itself adds the pixel's coordinates and clamps the sum to
+    // [lo, hi] (sampling_position below; the kernels that read a position once per head-query do this, the LDS-tile
+    // path is given positions a pass of its own has prepared).
+    int rel_heads;
+    float lo_x, hi_x, lo_y, hi_y;
 };
 
 // bytes the output views span (the last row ends with its data, not with its stride)
@@ -76,6 +83,27 @@ __device__ __forceinline__ void corner_weights(float x, float y, float &x0, floa
     w[1] = Tr::round(fx * gy);
     w[2] = Tr::round(gx * fy);
     w[3] = Tr::round(fx * fy);
+}
+
+// The sampling position of (pixel, head).  With relative positions this is what the attention layer and module
+// compute in four elementwise launches before the operator (models/attention_blocks.py:149-151 or 162-163: the
+// pixel's own coordinates are added in the tensor dtype -- coordinates beyond the dtype's exact integers round as
+// torch.arange in that dtype does; :45-59, :79: clamp to [r, size-1-r-1e-3] with the bounds rounded to the tensor
+// dtype; torch.clamp keeps NaN).
+template <typename T>
+__device__ __forceinline__ void sampling_position(const FwdArgs &A, long long pix, int head, float &x, float &y) {
+    typedef Traits<T> Tr;
+    const long long at = A.rel_heads == 1 ? pix : pix * A.h + head;
+    const T *p = (const T *)A.mo + at * 2;
+    x = Tr::to_f(p[0]);
+    y = Tr::to_f(p[1]);
+    if (A.rel_heads != 0) {
+        const int n = (int)(pix % A.N), py = n / A.W, px = n - py * A.W;
+        x = Tr::round(x + Tr::round((float)px));
+        y = Tr::round(y + Tr::round((float)py));
+        x = x != x ? x : fminf(fmaxf(x, Tr::round(A.lo_x)), Tr::round(A.hi_x));
+        y = y != y ? y : fminf(fmaxf(y, Tr::round(A.lo_y)), Tr::round(A.hi_y));
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -142,8 +170,8 @@ __global__ __launch_bounds__(256, R == 1 ? MA_FWD_WAVES : MA_FWD_WAVES_R2) void 
     const uint32_t kDead = 0xFFFFFF00u;      // beyond any buffer: the load returns zeros
 
     // sampling centre
-    const T *mo = (const T *)A.mo + (size_t)hq * 2;
-    const float x = Tr::to_f(mo[0]), y = Tr::to_f(mo[1]);
+    float x, y;
+    sampling_position<T>(A, pix, head, x, y);
     float x0, y0, w[4];
     corner_weights<T>(x, y, x0, y0, w);
     const int ix = centre_index(x0), iy = centre_index(y0);
@@ -344,8 +372,8 @@ __device__ __forceinline__ void fwd_generic_one(const FwdArgs &A, long long hq) 
     const long long pix = hq / A.h;
     const int head = (int)(hq - pix * A.h);
     const long long b = pix / A.N;
-    const T *mo = (const T *)A.mo + hq * 2;
-    const float x = Tr::to_f(mo[0]), y = Tr::to_f(mo[1]);
+    float x, y;
+    sampling_position<T>(A, pix, head, x, y);
     float x0, y0, w[4];
     corner_weights<T>(x, y, x0, y0, w);
     const int ix = centre_index(x0), iy = centre_index(y0);

@@ -72,7 +72,6 @@ __global__ __launch_bounds__(256, h16_waves(R, VPL)) void fwd_h16_kernel(FwdArgs
     const bool tail = slot >= npix;          // whole lane groups fall off the end together
     if (tail) slot = npix - 1;               // keep them in flight (DPP partners), store nothing
     const int pix = slot;
-    const int hq = pix * A.h + head;
     const bool carries = sub < Cfg::NVL;
     const bool live = carries && !tail;
     const int bN = (npix == A.N) ? 0 : (pix / A.N) * A.N;   // first pixel of this batch item
@@ -80,8 +79,8 @@ __global__ __launch_bounds__(256, h16_waves(R, VPL)) void fwd_h16_kernel(FwdArgs
     const uint32_t total_bytes = (uint32_t)(A.nhq / A.h) * row_bytes;
     const uint32_t chan_bytes = (uint32_t)(head * CH + sub * VPL * EPV) * 2u;
 
-    const half2_t xy = *(const half2_t *)((const T *)A.mo + (size_t)hq * 2);
-    const float x = (float)xy.x, y = (float)xy.y;
+    float x, y;
+    sampling_position<T>(A, pix, head, x, y);
     float x0, y0, w[4];
     corner_weights<T>(x, y, x0, y0, w);
     const int ix = centre_index(x0), iy = centre_index(y0);

@@ -64,9 +64,11 @@ def test_fused_entry_validates_before_any_gpu_call():
     import torch
     from matchattention_amd import fused_module_forward
     lib = _cabi.load()
-    # the workspace covers the sampling positions (2 values per head-query, rounded up to 256 bytes) plus the forward's own
-    n = lib.matchattn_forward_fused_workspace_bytes(1, 8, 8, 32, 4, 1, 1, _cabi.F16)
-    assert n == 1024 + lib.matchattn_forward_workspace_bytes(1, 8, 8, 32, 4, 1, 1, _cabi.F16)
+    # maps below the LDS-tile path's sizes need no scratch (the kernel adds the pixel grid and clamps itself); on that
+    # path the workspace covers the sampling positions (2 values per head-query) plus the forward's own
+    assert lib.matchattn_forward_fused_workspace_bytes(1, 8, 8, 32, 4, 1, 1, _cabi.F16) == 0
+    big = (1, 544, 960, 256, 8, 2, 2, _cabi.F16)
+    assert lib.matchattn_forward_fused_workspace_bytes(*big) == 544 * 960 * 8 * 2 * 2 + lib.matchattn_forward_workspace_bytes(*big) > 0
     assert lib.matchattn_forward_fused(None, 4, None, None, None, None, None, 0, None, 0, None, 0, 1, 8, 8, 32, 4, 1, 1, 1.0, 1, None) == 1
     assert b"null" in lib.matchattn_last_error()
     import ctypes
@@ -74,7 +76,7 @@ def test_fused_entry_validates_before_any_gpu_call():
     p = ctypes.addressof(host)
     assert lib.matchattn_forward_fused(p, 3, p, p, p, None, p, 0, p, 0, None, 0, 1, 8, 8, 32, 4, 1, 1, 1.0, 1, None) == 1
     assert b"position_heads" in lib.matchattn_last_error()
-    assert lib.matchattn_forward_fused(p, 4, p, p, p, None, p, 0, p, 0, None, 0, 1, 8, 8, 32, 4, 1, 1, 1.0, 1, None) == 2
+    assert lib.matchattn_forward_fused(p, 8, p, p, p, None, p, 0, p, 0, p, 16, 1, 544, 960, 256, 8, 2, 2, 1.0, 1, None) == 2
     assert b"workspace" in lib.matchattn_last_error()
     assert lib.matchattn_forward_fused(p, 0, p, p, p, None, p, -1, p, 0, None, 0, 1, 8, 8, 32, 4, 1, 1, 1.0, 1, None) == 1
     assert b"stride" in lib.matchattn_last_error()

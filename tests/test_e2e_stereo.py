@@ -5,13 +5,15 @@ Two measurements:
   * teacher-forced: the PyTorch operator drives the network and, at each of its 52 calls, the
     HIP operator is evaluated on the very same inputs -- parity at the real model shapes
     (Ch = 40/32/16/8, r = 2/2/1/1, self and cross) to the operator tolerances;
-  * free-running: both operators drive the network on their own.  A random-init network is
-    chaotic (floor() of the sampling centres, arg-max of the initial correlation, 26 layers that
-    divide the field by field_scale = 0.1; fields of several hundred px where fp16 spacing is
-    0.5 px), so the 0.05 px bound quoted for this configuration is below the network's own
-    sensitivity: a half-ulp perturbation of the PyTorch operator's outputs moves the final
-    disparity by as much.  The test therefore bounds the HIP-vs-PyTorch difference by that
-    measured noise floor and prints all figures."""
+  * free-running (a diagnostic, not a parity criterion): both operators drive the network on their
+    own.  The 0.05 px mean-disparity bound quoted for this configuration is UNPINNED here: it
+    presumes trained weights, and no checkpoint can be loaded.  A random-init network is chaotic
+    (floor() of the sampling centres, arg-max of the initial correlation, 26 layers that divide
+    the field by field_scale = 0.1; fields of several hundred px where fp16 spacing is 0.5 px):
+    a half-ulp perturbation of the PyTorch operator's own outputs moves the final disparity by
+    0.4-1 px.  The test prints the HIP-vs-PyTorch difference beside that measured self-noise of
+    the reference (several draws) and only checks that the former is of the latter's size; what
+    gates parity at the model's shapes is the teacher-forced test."""
 import pytest
 import torch
 
@@ -52,7 +54,7 @@ def test_operator_parity_at_every_call_of_the_model(hip_lib, dtype, tol):
     assert max(worst) <= tol
 
 
-def test_free_running_difference_is_at_the_noise_floor(hip_lib):
+def test_free_running_difference_is_of_the_size_of_the_references_own_noise(hip_lib):
     from matchattention_amd import MF_FusedForwardOps
     from matchattention_amd.workloads import make_stereo_pair
     hip_op = MF_FusedForwardOps()
