@@ -74,6 +74,17 @@ __global__ __launch_bounds__(256) void make_offsets_kernel(const T *rel, T *mo, 
 
 KernelTimer g_fwd_timer = {{false}, nullptr, nullptr};
 
+unsigned tile_grid(unsigned per_cu) {
+    static std::atomic<int> cus[64];                   // compute units per device index, 0 = not asked yet
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) n = cus[dev].load(std::memory_order_relaxed);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        if (dev >= 0 && dev < 64) cus[dev].store(n, std::memory_order_relaxed);
+    }
+    return (((unsigned)n * per_cu + 7u) / 8u) * 8u;
+}
+
 }  // namespace ma
 
 namespace {
@@ -267,7 +278,8 @@ ma::TileSort tile_sort_args(const ma::SortArgs &S, const TileLayout &tl, char *w
     T.count = S.count; T.rowtot = S.rowtot; T.per_head = S.per_head; T.perm = S.perm;
     T.defer = (uint8_t *)(ws + tl.defer_off); T.chunk_start = (int *)(ws + tl.chunk_off);
     T.chunk_item = (int2 *)(ws + tl.item_off); T.chunk_cap = tl.chunk_cap;
-    T.queue = S.per_head + 8;                          // inside the 256-byte flag block the sort zeroes
+    T.queue = S.per_head + ma::kFlagQueue;             // inside the 256-byte flag block the sort zeroes
+    T.xcd_bounds = S.per_head + ma::kFlagXcdBounds;
     T.bins_per_row = tl.sl.bins_per_row; T.nbins = tl.sl.nbins; T.nrows = tl.sl.nrows; T.rows_per_img = tl.sl.rows_per_img;
     T.L = S.L;
     return T;

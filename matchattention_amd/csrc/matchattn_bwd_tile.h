@@ -54,7 +54,11 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
     const int nitems = nchunks * nhg;
     const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
-    const int item_end = (int)((long long)nitems * (xcd + 1) >> 3);
+    // XCD x takes the x-th share of the work list (consecutive chunks, shares of equal cost: tile_chunks_kernel), the
+    // head groups of a chunk being neighbours in the item order; bounds read from scratch memory are clamped
+    const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
+    const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
+    (void)nitems;
     const bool per_head = *S.per_head != 0;
     // (the order of an item's prologue follows the forward kernel: staging addresses, the two index loads, the
     // staging loads, then the first pass's rows while the staging loads are in flight; the work-list entry is
@@ -65,16 +69,15 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
     (void)per_xcd;
     __shared__ int s_claim;
     int *const queue = S.queue + xcd;
-    const int xcd_start = (int)((long long)nitems * xcd >> 3);
     if (threadIdx.x == 0) s_claim = atomicAdd(queue, 2);
     __syncthreads();
     const int item0 = xcd_start + *(volatile int *)&s_claim;
     int item_next = item0 + 1;
 #else
-    const int item0 = (int)((long long)nitems * xcd >> 3) + (int)(blockIdx.x >> 3);
+    const int item0 = xcd_start + (int)(blockIdx.x >> 3);
 #endif
     int2 entry = int2{0, 0};
-    if (item0 < item_end) entry = S.chunk_item[item0 - (item0 / nchunks) * nchunks];
+    if (item0 < item_end) entry = S.chunk_item[item0 / nhg];
 #if MA_TILE_QUEUE
     for (int item = item0; item < item_end;) {
     int claim = 0;
@@ -82,7 +85,7 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
 #else
     for (int item = item0; item < item_end; item += per_xcd) {
 #endif
-        const int hgrp = item / nchunks;
+        const int hgrp = item - (item / nhg) * nhg;
         const int bin = clampi(entry.x, 0, S.nbins - 1), part = max(entry.y, 0);
         const int head = hgrp * HPG + hslot;
         int lo, hi;
@@ -133,7 +136,7 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
 #else
         const int item_n = min(item + per_xcd, item_end - 1);       // (the last item fetches its own entry again)
 #endif
-        const int2 entry_n = S.chunk_item[item_n - (item_n / nchunks) * nchunks];
+        const int2 entry_n = S.chunk_item[item_n / nhg];
 
         __syncthreads();                              // every wave is done with the previous tiles
 #pragma unroll

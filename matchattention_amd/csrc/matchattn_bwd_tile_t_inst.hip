@@ -23,8 +23,8 @@ template <int CH, int R>
 static int launch_bwd_tile(const BwdArgs &A, const TileSort &S, hipStream_t s) {
     typedef TileCfgT<T, CH, R, kTileW, kTileH, 1> Cfg;
     if (A.h % Cfg::HPG != 0) return -1;
-    hipLaunchKernelGGL(tile_chunks_kernel<0>, dim3(1), dim3(1024), 0, s, S, A.h, S.chunk_start);
-    const unsigned grid = 256u * 2u * (unsigned)kTileGridMult;     // persistent, a multiple of the 8 XCDs
+    launch_tile_chunks(S, A.h, Cfg::QPP, s);
+    const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);   // persistent: two workgroups fit a CU's LDS
     hipLaunchKernelGGL((bwd_tile_kernel<T, CH, R, kTileW, kTileH>), dim3(grid), dim3(kTileNT), 0, s, A, S);
     return (int)hipGetLastError();
 }

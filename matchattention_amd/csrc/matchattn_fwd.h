@@ -57,6 +57,7 @@ struct TileSort {
     int chunk_cap;
     int bins_per_row, nbins, nrows, rows_per_img, L;
     int *queue;            // [8] zero on entry: next unclaimed item of each XCD's share of the work list
+    int *xcd_bounds;       // [9] chunks [xcd_bounds[x], xcd_bounds[x + 1]) of the work list are XCD x's share (equal cost)
 };
 
 // Map the hardware workgroup id to a logical one so that each of the 8 XCDs

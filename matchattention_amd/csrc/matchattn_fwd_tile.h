@@ -109,15 +109,27 @@ __device__ __forceinline__ int tile_visit_order(const TileSort &S, int k) {
 }
 
 // chunk_start[bin] = number of chunks in the buckets visited before `bin` (exclusive scan in visiting order),
-// chunk_start[nbins] = all of them; chunk_item[c] = (bucket, index within the bucket) of chunk c.  A bucket has ceil(n / kTileCap) chunks, n being its largest population over the heads;
-// empty buckets have none.  One workgroup of 1024 threads.
-template <int Unused = 0>   // a template only so that several translation units may include this header
-__global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, int *chunk_start) {
+// chunk_start[nbins] = all of them; chunk_item[c] = (bucket, index within the bucket) of chunk c.  A bucket has
+// ceil(n / kTileCap) chunks, n being its largest population over the heads; empty buckets have none.
+// xcd_bounds[x] = first chunk of XCD x's share of the list: the shares are consecutive runs of equal cost, a chunk
+// being priced at its passes (ceil(population / qpp)) plus kChunkFixedCost for staging its tiles.  (Shares of equal
+// length differ in cost by the chunks of the border tiles, which collect the clamped centres of a whole margin
+// of the image and are full, while interior chunks hold a tile's own queries.)  One workgroup of 1024 threads.
+#ifndef MA_TILE_FIXED_COST
+#define MA_TILE_FIXED_COST 1
+#endif
+constexpr int kChunkFixedCost = MA_TILE_FIXED_COST;
+// (A template so that every translation unit may include this header; only launch_tile_chunks names it, so one
+// translation unit alone holds the kernel.)
+template <int Unused = 0>
+__global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, int *chunk_start, int qpp) {
     __shared__ int part[1024];
+    __shared__ int cost_part[1024];
     const int per = (S.nbins + 1023) / 1024;
     const int b0 = min((int)threadIdx.x * per, S.nbins), b1 = min(b0 + per, S.nbins);
     const int nh = *S.per_head ? h : 1;
-    int sum = 0;
+    const int full_cost = (kTileCap + qpp - 1) / qpp + kChunkFixedCost;
+    int sum = 0, cost_sum = 0;
     for (int pos = b0; pos < b1; ++pos) {
         const int bin = tile_visit_order(S, pos);
         int n = 0;
@@ -127,27 +139,47 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
             n = max(n, hi - lo);
         }
         const int c = (n + kTileCap - 1) / kTileCap;
-        chunk_start[bin] = c;
+        chunk_start[bin] = n;                         // (population for now: the second walk prices the chunks from it)
         sum += c;
+        const int rem = n - (n / kTileCap) * kTileCap;
+        cost_sum += (n / kTileCap) * full_cost + (rem ? (rem + qpp - 1) / qpp + kChunkFixedCost : 0);
     }
     part[threadIdx.x] = sum;
+    cost_part[threadIdx.x] = cost_sum;
     __syncthreads();
     for (int d = 1; d < 1024; d <<= 1) {          // Hillis-Steele inclusive scan of the partial sums
         const int v = (int)threadIdx.x >= d ? part[threadIdx.x - d] : 0;
+        const int cv = (int)threadIdx.x >= d ? cost_part[threadIdx.x - d] : 0;
         __syncthreads();
         part[threadIdx.x] += v;
+        cost_part[threadIdx.x] += cv;
         __syncthreads();
     }
+    const long long total_cost = cost_part[1023];
     int run = part[threadIdx.x] - sum;
+    long long cost_run = cost_part[threadIdx.x] - cost_sum;
     for (int pos = b0; pos < b1; ++pos) {
         const int bin = tile_visit_order(S, pos);
-        const int c = chunk_start[bin];
+        const int n = chunk_start[bin];
+        const int c = (n + kTileCap - 1) / kTileCap;
         chunk_start[bin] = run;
         // the work list itself: entry = (bucket, which chunk of it), so that a workgroup finds its item with one load
-        for (int k = 0; k < c && run + k < S.chunk_cap; ++k) S.chunk_item[run + k] = int2{bin, k};
+        for (int k = 0; k < c; ++k) {
+            if (run + k < S.chunk_cap) S.chunk_item[run + k] = int2{bin, k};
+            const int pop = min(n - k * kTileCap, kTileCap);
+            const long long after = cost_run + (pop + qpp - 1) / qpp + kChunkFixedCost;
+            // share x starts behind the chunk in which the running cost reaches x eighths of the total
+            for (int x = (int)(cost_run * 8 / total_cost) + 1; x <= 7 && x * total_cost <= after * 8; ++x)
+                S.xcd_bounds[x] = min(run + k + 1, S.chunk_cap);
+            cost_run = after;
+        }
         run += c;
     }
-    if (threadIdx.x == 1023) chunk_start[S.nbins] = min(part[1023], S.chunk_cap);
+    if (threadIdx.x == 1023) {
+        chunk_start[S.nbins] = min(part[1023], S.chunk_cap);
+        S.xcd_bounds[0] = 0;
+        S.xcd_bounds[8] = min(part[1023], S.chunk_cap);
+    }
 }
 
 template <int CH, int R, int TW, int TH, int VPL>
@@ -202,8 +234,8 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 
     // ---- work items: (head group, chunk of at most kTileCap queries per head of one bucket) ----------
     // A fixed grid of persistent workgroups.  Workgroup ids are dealt round-robin to the 8 XCDs; XCD x takes the
-    // x-th eighth of the items, which are ordered by head group, then tile, so that one L2 sees one head group
-    // of one band of neighbouring tiles.  Within that share the workgroups claim items from a counter
+    // x-th share of the work list (consecutive chunks, shares of equal cost: tile_chunks_kernel), so that one L2
+    // sees one band of neighbouring tiles.  Within that share the workgroups claim items from a counter
     // (MA_TILE_QUEUE; a fixed stride without it).
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
     const int nitems = nchunks * nhg;
@@ -213,7 +245,10 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     auto item_chunk = [&](int it) __attribute__((always_inline)) { return it / nhg; };
     auto item_hgrp = [&](int it) __attribute__((always_inline)) { return it - (it / nhg) * nhg; };
     const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
-    const int item_end = (int)((long long)nitems * (xcd + 1) >> 3);
+    // (bounds read from scratch memory are clamped before they become indices)
+    const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
+    const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
+    (void)nitems;
     const bool per_head = *S.per_head != 0;
     // Memory round trips of an item, in order: its work-list entry (fetched one item ahead), the bounds of its
     // bucket, the pixel indices of its first two passes -- issued before the staging loads, which return
@@ -227,13 +262,12 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     (void)per_xcd;
     __shared__ int s_claim;
     int *const queue = S.queue + xcd;
-    const int xcd_start = (int)((long long)nitems * xcd >> 3);
     if (threadIdx.x == 0) s_claim = atomicAdd(queue, 2);
     __syncthreads();
     const int item0 = xcd_start + *(volatile int *)&s_claim;
     int item_next = item0 + 1;
 #else
-    const int item0 = (int)((long long)nitems * xcd >> 3) + (int)(blockIdx.x >> 3);
+    const int item0 = xcd_start + (int)(blockIdx.x >> 3);
 #endif
     int2 entry = int2{0, 0};
     if (item0 < item_end) entry = S.chunk_item[item_chunk(item0)];

@@ -6,6 +6,9 @@ namespace ma {
 
 const int kTileLog2[2] = {kTileWLog2, kTileHLog2};
 const int kTileCapHost = kTileCap;
+void launch_tile_chunks(const TileSort &S, int h, int queries_per_pass, hipStream_t s) {
+    hipLaunchKernelGGL(tile_chunks_kernel<0>, dim3(1), dim3(1024), 0, s, S, h, S.chunk_start, queries_per_pass > 0 ? queries_per_pass : 64);
+}
 
 #ifndef MA_TILE_VPL
 #define MA_TILE_VPL 2
@@ -18,9 +21,9 @@ static int launch_tile(const FwdArgs &A, const TileSort &S, hipStream_t s) {
     FwdArgs B = A;
     const int nhg = A.h / Cfg::HPG;
     (void)nhg;
-    hipLaunchKernelGGL(tile_chunks_kernel<0>, dim3(1), dim3(1024), 0, s, S, A.h, S.chunk_start);
-    // persistent grid: a few workgroups per CU (256 CUs, two fit a CU's LDS), a multiple of the 8 XCDs
-    const unsigned grid = 256u * 2u * (unsigned)kTileGridMult;
+    launch_tile_chunks(S, A.h, Cfg::QPP, s);
+    // persistent grid: a few workgroups per CU, a multiple of the 8 XCDs
+    const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);   // persistent: two workgroups fit a CU's LDS
     timer_mark(false, s);
     hipLaunchKernelGGL((fwd_h16_tile_kernel<CH, R, kTileW, kTileH, VPL>), dim3(grid), dim3(kTileNT), 0, s, B, S);
     timer_mark(true, s);

@@ -26,8 +26,8 @@ static int launch_tile(const FwdArgs &A, const TileSort &S, hipStream_t s) {
     constexpr int VPL = CH * (int)sizeof(T) >= 32 ? 2 : 1;            // vectors per lane
     typedef TileCfgT<T, CH, R, kTileW, kTileH, VPL> Cfg;
     if (A.h % Cfg::HPG != 0) return -1;
-    hipLaunchKernelGGL(tile_chunks_kernel<0>, dim3(1), dim3(1024), 0, s, S, A.h, S.chunk_start);
-    const unsigned grid = 256u * 2u * (unsigned)kTileGridMult;     // persistent, a multiple of the 8 XCDs
+    launch_tile_chunks(S, A.h, Cfg::QPP, s);
+    const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);   // persistent: two workgroups fit a CU's LDS
     timer_mark(false, s);
     hipLaunchKernelGGL((fwd_tile_kernel<T, CH, R, kTileW, kTileH, VPL>), dim3(grid), dim3(kTileNT), 0, s, A, S);
     timer_mark(true, s);

@@ -34,6 +34,15 @@ extern KernelTimer g_fwd_timer;
 inline void timer_mark(bool end, hipStream_t s) {
     if (g_fwd_timer.on) (void)hipEventRecord(end ? g_fwd_timer.after : g_fwd_timer.before, s);
 }
+// Size of the persistent grid of the LDS-tile kernels: `per_cu` workgroups for every compute unit of the current device
+// (asked from the runtime once per device), rounded up to a multiple of the 8 XCDs the kernels' work split assumes
+// (workgroup i runs on XCD i mod 8; on a part with another XCD count the split still covers every item, each
+// workgroup claiming from the counter of "its" eighth, only the L2 locality it aims for is lost).
+unsigned tile_grid(unsigned per_cu);
+// Builds the work list of the LDS-tile kernels (tile_chunks_kernel); queries_per_pass is the number of queries per head the
+// consuming kernel takes from a chunk at a time (prices a chunk for the split of the list among the XCDs).  Defined once, beside the fp16 forward tile kernel:
+// a second copy in another translation unit would be a second device kernel of the same name.
+void launch_tile_chunks(const TileSort &S, int h, int queries_per_pass, hipStream_t s);
 extern const int kTileLog2[2];       // log2 of the tile width and height the kernel was built for
 extern const int kTileCapHost;       // queries per head in one work item of that kernel
 

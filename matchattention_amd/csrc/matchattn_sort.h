@@ -38,9 +38,16 @@ struct SortArgs {
     int *perm;             // [h][L]
     int *centre;           // optional [h][L]: centre of the entry at the same position, (cy << 16) | (cx & 0xffff),
                            //   each saturated to int16 (enough to decide which taps reach a key); or null
-    int *per_head;         // [2] (zero on entry): [0] heads need their own permutation, [1] number of
-                           //     (pixel, head) pairs whose target is not next to their left neighbour's
+    int *per_head;         // the 256-byte flag block (zero on entry, layout below): [kFlagPerHead] heads need their own
+                           //     permutation, [kFlagIncoherent] number of (pixel, head) pairs whose target is not next to
+                           //     their left neighbour's
 };
+// Words of the flag block the sort zeroes with its counters (64 ints).  The LDS-tile kernels keep their work
+// counters, one per XCD, in the same block (TileSort::queue = per_head + kFlagQueue), and the work list's split among
+// the XCDs (TileSort::xcd_bounds = per_head + kFlagXcdBounds).
+constexpr int kFlagPerHead = 0, kFlagIncoherent = 1, kFlagQueue = 8, kFlagQueueSlots = 8, kFlagXcdBounds = 16, kFlagXcdBoundSlots = 9,
+              kFlagWords = 64;
+static_assert(kFlagQueue + kFlagQueueSlots <= kFlagXcdBounds && kFlagXcdBounds + kFlagXcdBoundSlots <= kFlagWords, "flag block layout");
 
 __device__ __forceinline__ void load_xy(const void *mo, int dtype, size_t idx, float &x, float &y) {
     if (dtype == 0) {
@@ -93,7 +100,7 @@ __device__ __forceinline__ int target_bin(const SortArgs &S, int pix, float x, f
 // called coherent when a pixel's target sits next to its left neighbour's (per head); the ordering is
 // used when more than 1/8 of the (pixel, head) pairs are not (decided on the device: no host round trip).
 __device__ __forceinline__ bool sort_useful(const SortArgs &S) {
-    return S.force || (long long)S.per_head[1] * 8 > (long long)S.L * S.h;
+    return S.force || (long long)S.per_head[kFlagIncoherent] * 8 > (long long)S.L * S.h;
 }
 
 // One thread per (pixel, head) and step of a grid-stride loop: the loads of a wavefront are adjacent, and a
@@ -151,11 +158,11 @@ __global__ __launch_bounds__(256) void sort_probe_kernel(SortArgs S) {
     __syncthreads();
     if (threadIdx.x == 0) {
         const int tn = part_n[0] + part_n[1] + part_n[2] + part_n[3];
-        if (tn) atomicAdd(&S.per_head[1], tn);
+        if (tn) atomicAdd(&S.per_head[kFlagIncoherent], tn);
         // (the others look first: one workgroup setting the flag is enough)
         if ((part_d[0] | part_d[1] | part_d[2] | part_d[3]) &&
-            __hip_atomic_load(&S.per_head[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
-            atomicOr(&S.per_head[0], 1);
+            __hip_atomic_load(&S.per_head[kFlagPerHead], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+            atomicOr(&S.per_head[kFlagPerHead], 1);
     }
 }
 
