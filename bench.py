@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 # (see profiles/): filled in from the committed counter summary, None when not measured.
 # keyed by (workload, first part of the kernel name that ran)
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg3_cross", "fwd_tile_f16"): 2144699392,    # LDS-tile kernel: 2.0 x 730769 KiB fetched + 632895 KiB written
+    ("cfg3_cross", "fwd_tile_f16"): 1872608256,    # LDS-tile kernel: 2.0 x 605521 KiB fetched + 617677 KiB written
     ("cfg3_cross", "fwd_tiled_f16"): 1470390272,   # direct-gather kernel: 2.0 x 424204 KiB fetched + 587520 KiB written
     ("cfg3_cross", "fwd_tile_f32"): 4541189120,    # fp32 LDS-tile kernel: 2.0 x 1581641 KiB fetched + 1271473 KiB written
 }
@@ -285,7 +285,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--workload", default="cfg3_cross")
     ap.add_argument("--direct", action="store_true",
                     help="time the direct-gather forward kernel instead of the LDS-tile path (forward_lds=0)")
