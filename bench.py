@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 MEASURED_TRAFFIC_BYTES = {
     ("cfg3_cross", "fwd_tile_f16"): 1872608256,    # LDS-tile kernel: 2.0 x 605521 KiB fetched + 617677 KiB written
     ("cfg3_cross", "fwd_tiled_f16"): 1470390272,   # direct-gather kernel: 2.0 x 424204 KiB fetched + 587520 KiB written
-    ("cfg3_cross", "fwd_tile_f32"): 4541189120,    # fp32 LDS-tile kernel: 2.0 x 1581641 KiB fetched + 1271473 KiB written
+    ("cfg3_cross", "fwd_tile_f32"): 3778794496,    # fp32 LDS-tile kernel: 2.0 x 1233603 KiB fetched + 1223023 KiB written
 }
 
 
