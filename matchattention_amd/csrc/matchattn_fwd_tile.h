@@ -72,10 +72,9 @@ constexpr int kTileGridMult = MA_TILE_GRID_MULT;
 #define MA_TILE_QUEUE 1
 #endif
 
-// [lo, hi) of bucket `bin` in the bucket order of head `src`, clamped so that values read from scratch
-// memory never become addresses unchecked
-__device__ __forceinline__ void bucket_bounds(const TileSort &S, int src, int bin, int &lo, int &hi) {
-    const int row = bin / S.bins_per_row, tx = bin - row * S.bins_per_row;
+// [lo, hi) of bucket `bin` (tile row `row` over all images, tile column `tx`) in the bucket order of head `src`,
+// clamped so that values read from scratch memory never become addresses unchecked
+__device__ __forceinline__ void bucket_bounds_at(const TileSort &S, int src, int bin, int row, int tx, int &lo, int &hi) {
     // four independent loads (both candidates for the end are fetched, then one is chosen): one latency
     const int row_start = S.rowtot[src * S.nrows + row];
     const int next_row = S.rowtot[src * S.nrows + min(row + 1, S.nrows - 1)];
@@ -86,39 +85,61 @@ __device__ __forceinline__ void bucket_bounds(const TileSort &S, int src, int bi
     lo = clampi(lo, 0, S.L);
     hi = clampi(hi, lo, S.L);
 }
+__device__ __forceinline__ void bucket_bounds(const TileSort &S, int src, int bin, int &lo, int &hi) {
+    const int row = bin / S.bins_per_row;
+    bucket_bounds_at(S, src, bin, row, bin - row * S.bins_per_row, lo, hi);
+}
 
 // Order in which the work list visits the tiles of an image: strips of kTileStrip tile columns, each walked row by
 // row from the top.  The workgroups of an XCD take consecutive items, so the tiles in flight form a block about as
 // tall as it is wide and the K/V rows a tile shares with the tile below it are still in that XCD's L2 when the
 // tile below is staged (in row-major order a whole tile row -- more than the L2 holds, with the query, output
 // and attention streams of its items -- passes in between, and the vertical halo is fetched from memory again).
+// TileWalk stands at one position of that order and steps to the next without a division (the one workgroup that
+// builds the work list is bound by its integer arithmetic: the position -> tile formula costs five divisions).
 #ifndef MA_TILE_STRIP
 #define MA_TILE_STRIP 8
 #endif
 constexpr int kTileStrip = MA_TILE_STRIP;
-__device__ __forceinline__ int tile_visit_order(const TileSort &S, int k) {
-    if (kTileStrip <= 0 || S.bins_per_row <= kTileStrip) return k;
-    const int per_img = S.rows_per_img * S.bins_per_row;
-    const int img = k / per_img, kk = k - img * per_img;
-    const int nfull = S.bins_per_row / kTileStrip;
-    const int strip = min(kk / (S.rows_per_img * kTileStrip), nfull);
-    const int w = strip < nfull ? kTileStrip : S.bins_per_row - nfull * kTileStrip;
-    const int within = kk - strip * S.rows_per_img * kTileStrip;
-    const int r = within / w, c = strip * kTileStrip + (within - r * w);
-    return (img * S.rows_per_img + r) * S.bins_per_row + c;
-}
+struct TileWalk {
+    int img, strip, r, c, w;      // image, strip, tile row within the image, column within the strip, the strip's width
+    int nfull, last_w, rows, bpr;
+    __device__ __forceinline__ TileWalk(const TileSort &S, int k) {
+        rows = S.rows_per_img; bpr = S.bins_per_row;
+        const bool strips = kTileStrip > 0 && bpr > kTileStrip;
+        nfull = strips ? bpr / kTileStrip : 0;                 // (without strips: one strip as wide as the image)
+        last_w = bpr - nfull * kTileStrip;
+        const int per_img = rows * bpr;
+        img = k / per_img;
+        const int kk = k - img * per_img;
+        strip = strips ? min(kk / (rows * kTileStrip), nfull) : 0;
+        w = strip < nfull ? kTileStrip : last_w;
+        const int within = kk - strip * rows * kTileStrip;
+        r = within / max(w, 1);
+        c = within - r * w;
+    }
+    __device__ __forceinline__ int row() const { return img * rows + r; }
+    __device__ __forceinline__ int col() const { return strip * kTileStrip + c; }
+    __device__ __forceinline__ int bin() const { return row() * bpr + col(); }
+    __device__ __forceinline__ void next() {
+        if (++c < w) return;
+        c = 0;
+        if (++r < rows) return;
+        r = 0;
+        ++strip;
+        if (strip > nfull || (strip == nfull && last_w == 0)) { strip = 0; ++img; }
+        w = strip < nfull ? kTileStrip : last_w;
+    }
+};
 
 // chunk_start[bin] = number of chunks in the buckets visited before `bin` (exclusive scan in visiting order),
 // chunk_start[nbins] = all of them; chunk_item[c] = (bucket, index within the bucket) of chunk c.  A bucket has
 // ceil(n / kTileCap) chunks, n being its largest population over the heads; empty buckets have none.
 // xcd_bounds[x] = first chunk of XCD x's share of the list: the shares are consecutive runs of equal cost, a chunk
-// being priced at its passes (ceil(population / qpp)) plus kChunkFixedCost for staging its tiles.  (Shares of equal
+// being priced at kPassCost per pass (ceil(population / qpp) passes) plus kChunkFixedCost for staging its tiles.  (Shares of equal
 // length differ in cost by the chunks of the border tiles, which collect the clamped centres of a whole margin
 // of the image and are full, while interior chunks hold a tile's own queries.)  One workgroup of 1024 threads.
-#ifndef MA_TILE_FIXED_COST
-#define MA_TILE_FIXED_COST 1
-#endif
-constexpr int kChunkFixedCost = MA_TILE_FIXED_COST;
+constexpr int kPassCost = 2, kChunkFixedCost = 1;     // (measured at cfg3/cfg4: 1+1 and 4+3 within 1 % of 2+1, 1+0 and 2+3 1.5 % off)
 // (A template so that every translation unit may include this header; only launch_tile_chunks names it, so one
 // translation unit alone holds the kernel.)
 template <int Unused = 0>
@@ -128,21 +149,55 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
     const int per = (S.nbins + 1023) / 1024;
     const int b0 = min((int)threadIdx.x * per, S.nbins), b1 = min(b0 + per, S.nbins);
     const int nh = *S.per_head ? h : 1;
-    const int full_cost = (kTileCap + qpp - 1) / qpp + kChunkFixedCost;
-    int sum = 0, cost_sum = 0;
-    for (int pos = b0; pos < b1; ++pos) {
-        const int bin = tile_visit_order(S, pos);
+    const int full_cost = (kTileCap + qpp - 1) / qpp * kPassCost + kChunkFixedCost;
+    auto population = [&](const TileWalk &at) __attribute__((always_inline)) {
         int n = 0;
         for (int hd = 0; hd < nh; ++hd) {
             int lo, hi;
-            bucket_bounds(S, hd, bin, lo, hi);
+            bucket_bounds_at(S, hd, at.bin(), at.row(), at.col(), lo, hi);
             n = max(n, hi - lo);
         }
-        const int c = (n + kTileCap - 1) / kTileCap;
-        chunk_start[bin] = n;                         // (population for now: the second walk prices the chunks from it)
-        sum += c;
-        const int rem = n - (n / kTileCap) * kTileCap;
-        cost_sum += (n / kTileCap) * full_cost + (rem ? (rem + qpp - 1) / qpp + kChunkFixedCost : 0);
+        return n;
+    };
+    auto price = [&](int n, int &chunks, int &cost) __attribute__((always_inline)) {
+        const int full = n / kTileCap, rem = n - full * kTileCap;
+        chunks += full + (rem ? 1 : 0);
+        cost += full * full_cost + (rem ? (rem + qpp - 1) / qpp * kPassCost + kChunkFixedCost : 0);
+    };
+    // Up to kChunkKeep buckets of a thread stay in registers -- tile and population, the populations of head 0 fetched by
+    // loads that do not depend on one another: one memory round trip instead of one per bucket, and the second walk reads
+    // nothing.  Larger maps park the populations in chunk_start between the walks.
+    constexpr int kChunkKeep = 4;
+    const bool keep = per <= kChunkKeep;
+    int kept_bin[kChunkKeep], kept_n[kChunkKeep];
+    int sum = 0, cost_sum = 0;
+    if (b0 < b1) {
+        TileWalk at(S, b0);
+        if (keep) {
+            int lo[kChunkKeep], hi[kChunkKeep];
+            TileWalk tile[kChunkKeep] = {at, at, at, at};
+#pragma unroll
+            for (int i = 0; i < kChunkKeep; ++i) {
+                tile[i] = at;
+                kept_bin[i] = at.bin();
+                if (i + 1 < per) at.next();               // (uniform; past the thread's last bucket the tile repeats and is masked below)
+            }
+#pragma unroll
+            for (int i = 0; i < kChunkKeep; ++i) bucket_bounds_at(S, 0, kept_bin[i], tile[i].row(), tile[i].col(), lo[i], hi[i]);
+#pragma unroll
+            for (int i = 0; i < kChunkKeep; ++i) {
+                kept_n[i] = hi[i] - lo[i];
+                if (nh > 1) kept_n[i] = max(kept_n[i], population(tile[i]));
+                if (b0 + i >= b1) kept_n[i] = 0;
+                price(kept_n[i], sum, cost_sum);
+            }
+        } else {
+            for (int pos = b0; pos < b1; ++pos, at.next()) {
+                const int n = population(at);
+                chunk_start[at.bin()] = n;                // (population for now: the second walk prices the chunks from it)
+                price(n, sum, cost_sum);
+            }
+        }
     }
     part[threadIdx.x] = sum;
     cost_part[threadIdx.x] = cost_sum;
@@ -158,22 +213,31 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
     const long long total_cost = cost_part[1023];
     int run = part[threadIdx.x] - sum;
     long long cost_run = cost_part[threadIdx.x] - cost_sum;
-    for (int pos = b0; pos < b1; ++pos) {
-        const int bin = tile_visit_order(S, pos);
-        const int n = chunk_start[bin];
+    int next_share = total_cost > 0 ? (int)(cost_run * 8 / total_cost) + 1 : 8;     // first share bound not yet behind this thread
+    // the work list itself: entry = (bucket, which chunk of it), so that a workgroup finds its item with one load
+    auto emit = [&](int bin, int n) __attribute__((always_inline)) {
         const int c = (n + kTileCap - 1) / kTileCap;
         chunk_start[bin] = run;
-        // the work list itself: entry = (bucket, which chunk of it), so that a workgroup finds its item with one load
         for (int k = 0; k < c; ++k) {
             if (run + k < S.chunk_cap) S.chunk_item[run + k] = int2{bin, k};
             const int pop = min(n - k * kTileCap, kTileCap);
-            const long long after = cost_run + (pop + qpp - 1) / qpp + kChunkFixedCost;
+            const long long after = cost_run + (pop + qpp - 1) / qpp * kPassCost + kChunkFixedCost;
             // share x starts behind the chunk in which the running cost reaches x eighths of the total
-            for (int x = (int)(cost_run * 8 / total_cost) + 1; x <= 7 && x * total_cost <= after * 8; ++x)
-                S.xcd_bounds[x] = min(run + k + 1, S.chunk_cap);
+            for (; next_share <= 7 && next_share * total_cost <= after * 8; ++next_share)
+                S.xcd_bounds[next_share] = min(run + k + 1, S.chunk_cap);
             cost_run = after;
         }
         run += c;
+    };
+    if (b0 < b1) {
+        if (keep) {
+#pragma unroll
+            for (int i = 0; i < kChunkKeep; ++i)
+                if (b0 + i < b1) emit(kept_bin[i], kept_n[i]);
+        } else {
+            TileWalk at(S, b0);
+            for (int pos = b0; pos < b1; ++pos, at.next()) emit(at.bin(), chunk_start[at.bin()]);
+        }
     }
     if (threadIdx.x == 1023) {
         chunk_start[S.nbins] = min(part[1023], S.chunk_cap);

@@ -119,6 +119,7 @@ __global__ __launch_bounds__(256) void sort_probe_kernel(SortArgs S) {
     // by integer division, not by its loads)
     const uint32_t total32 = (uint32_t)total, stride = gridDim.x * 256u, uh = (uint32_t)S.h;
     const int hshift = (uh & (uh - 1)) == 0 ? __builtin_ctz(uh) : -1;
+    const bool from_lane = hshift >= 0 && uh <= 64u;
     for (uint32_t base = blockIdx.x * 256u; base < total32; base += stride * UNR) {
         float x[UNR], y[UNR], xl[UNR], yl[UNR], x0[UNR], y0[UNR];
         bool in[UNR], other[UNR];
@@ -130,11 +131,21 @@ __global__ __launch_bounds__(256) void sort_probe_kernel(SortArgs S) {
             const uint32_t hd = hshift >= 0 ? (at & (uh - 1)) : at % uh;
             other[u] = in[u] && hd != 0;
             load_xy_as<DT>(S.mo, (size_t)at, x[u], y[u]);
-            load_xy_as<DT>(S.mo, (size_t)(at - hd), x0[u], y0[u]);
+            if (!from_lane) load_xy_as<DT>(S.mo, (size_t)(at - hd), x0[u], y0[u]);
             xl[u] = x[u] - 1.0f; yl[u] = y[u];
             if (!S.force) {
                 const uint32_t pix = hshift >= 0 ? at >> hshift : at / uh;
                 if (pix % (uint32_t)S.W != 0) load_xy_as<DT>(S.mo, (size_t)(at - uh), xl[u], yl[u]);
+            }
+        }
+        if (from_lane) {
+            // head 0 of a lane's pixel sits h-aligned in the same wavefront (indices are lane-aligned: base and stride
+            // are multiples of 256): its position comes from that lane's registers, not from a second load
+            const int src = (int)(threadIdx.x & 63u & ~(uh - 1u));
+#pragma unroll
+            for (int u = 0; u < UNR; ++u) {
+                x0[u] = __shfl(x[u], src);
+                y0[u] = __shfl(y[u], src);
             }
         }
 #pragma unroll
@@ -143,10 +154,13 @@ __global__ __launch_bounds__(256) void sort_probe_kernel(SortArgs S) {
             // exact index: heads share an index only if their (unclamped) centres coincide, because
             // the stored centre of head 0 then stands for every head; coarse ordering: same cell suffices
             // (same pixel, so the same batch item)
-            if (other[u])
+            // (equal positions need no cells: with shared positions, the usual case, the wavefront skips the arithmetic
+            // that otherwise bounds this kernel)
+            const bool unequal = other[u] && !(x[u] == x0[u] && y[u] == y0[u]);
+            if (__builtin_amdgcn_ballot_w64(unequal) != 0 && unequal)
                 differ = differ || (S.bin_shift == 0 ? pack_centre(x[u], y[u]) != pack_centre(x0[u], y0[u])
                                                      : target_cell(S, x[u], y[u]) != target_cell(S, x0[u], y0[u]));
-            n += __builtin_popcountll(__builtin_amdgcn_ballot_w64(incoherent));
+            if (!S.force) n += __builtin_popcountll(__builtin_amdgcn_ballot_w64(incoherent));
         }
     }
     const int wave = threadIdx.x >> 6;
