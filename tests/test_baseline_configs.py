@@ -87,3 +87,62 @@ def test_large_maps_forward_whole_map(hip_lib, name):
     want_out, want_attn = O.forward_chunked(*cpu, H, W, [wl.r, wl.r], wl.scale, rows_per_chunk=8)
     check_err(attn, want_attn, TOL[dt], f"{name} fwd attn f16")
     check_err(out, want_out, TOL[dt], f"{name} fwd out f16")
+
+
+def test_map_with_more_tiles_than_a_thread_keeps(hip_lib):
+    """A map of 96 x 88 = 8 448 tiles of 16 x 8 pixels: the work-list kernel's threads then take nine buckets each and
+    park their populations in scratch memory between the two walks (up to four stay in registers, which is what the
+    benchmark shapes exercise), two images so that the tile walk crosses an image boundary inside a thread's run, a
+    last strip narrower than the others (88 = 10 x 8 + 8 is even; 1 400 pixels = 87.5 tiles gives the ragged edge).
+    Forward against the oracle on bands of query rows at the top, across the image boundary and at the bottom, the
+    whole map against the direct-gather kernel, and the tile kernel must have served (nearly) every query."""
+    from matchattention_amd import _cabi
+    torch.manual_seed(11)
+    B, H, W, h, Ch, r = 2, 384, 1400, 4, 16, 2
+    N, C = H * W, h * Ch
+    dev = "cuda"
+    q, k, v = (torch.randn(B, N, C, device=dev, dtype=torch.float16) for _ in range(3))
+    coords = O.init_coords(B, H, W).view(B, N, 1, 2).to(dev)
+    rel = torch.zeros(B, N, h, 2, device=dev)
+    rel[..., 0] = -torch.rand(B, N, 1, device=dev) * 96 + torch.randn(B, N, h, device=dev) * 0.7     # per-head positions
+    rel[..., 1] = torch.randn(B, N, h, device=dev) * 2.0
+    mo = O.clamp_max_offset((coords + rel).half(), H, W, [r, r]).contiguous()
+    scale = Ch ** -0.5
+    nbins = B * ((H + 7) // 8) * ((W + 15) // 16)
+    assert nbins > 4 * 1024
+    deferred = []
+    _cabi.set_option("forward_lds", 1)
+    try:
+        out, attn = hip_forward(hip_lib, mo, q, k, v, H, W, r, scale, deferred=deferred)
+        assert _cabi.last_forward_kernel().startswith("fwd_tile_")
+    finally:
+        _cabi.set_option("forward_lds", -1)
+    assert 0 <= deferred[0] < 0.001 * B * N * h, deferred
+    _cabi.set_option("forward_lds", 0)
+    try:
+        out_d, attn_d = hip_forward(hip_lib, mo, q, k, v, H, W, r, scale)
+    finally:
+        _cabi.set_option("forward_lds", -1)
+    check_err(out, out_d, TOL[torch.float16], "many tiles: tile vs direct out f16")
+    check_err(attn, attn_d, TOL[torch.float16], "many tiles: tile vs direct attn f16")
+    for y0 in (0, H - 8, 2 * H - 16):                       # rows of the stacked images: top, image boundary, bottom
+        b, y = divmod(y0, H)
+        rows = min(16, H - y)
+        sl = slice(y * W, (y + rows) * W)
+        want_out, want_attn = _oracle_rows(mo[b:b + 1, sl].cpu(), q[b:b + 1, sl].cpu(), k[b:b + 1].cpu(), v[b:b + 1].cpu(),
+                                           H, W, r, scale)
+        check_err(out[b:b + 1, sl].cpu(), want_out, TOL[torch.float16], "many tiles fwd out f16")
+        check_err(attn[b:b + 1, sl].cpu(), want_attn, TOL[torch.float16], "many tiles fwd attn f16")
+
+
+def _oracle_rows(mo, q, k, v, H, W, r, scale):
+    """The oracle's forward for a band of queries (mo [B,n,h,2], q [B,n,C]) against the whole K and V [B,N,C]:
+    the steps of oracle.mat_oracle.forward_chunked on one band."""
+    B, n, C = q.shape
+    h = mo.size(2)
+    k4, v4 = k.view(B, k.size(1), h, -1), v.view(B, v.size(1), h, -1)
+    with torch.no_grad():
+        idx = O.tap_indices(torch.floor(mo).to(torch.int32), [r, r], H, W)
+        lg = O.window_logits(q.reshape(B, n, h, -1), k4, idx) * scale
+        a = O.bilinear_softmax(lg, O.corner_weights(mo), [r, r])
+        return O.aggregate(v4, a, idx), a
