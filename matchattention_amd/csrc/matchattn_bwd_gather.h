@@ -39,10 +39,11 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
 
     const int sub = threadIdx.x % LPH;
     // each XCD (workgroup ids are dealt to them round-robin) takes one contiguous band of keys: neighbouring
-    // keys share most of their candidate queries, which then meet in one L2.  Not with an index per head: the
-    // heads of a key then walk eight unrelated lists, and dealing the blocks round-robin measured 4 % faster
-    // (2 x 384 x 384, 8 heads, offsets N(0, 24 px) per head: 3.22 -> 3.09 ms for the whole backward).
-    const unsigned blk = logical_block(blockIdx.x, gridDim.x, A.xcd_swizzle && A.per_head[0] == 0);
+    // keys share most of their candidate queries, which then meet in one L2.  Not with an index per head and 16-bit
+    // tensors: the heads of a key then walk eight unrelated lists, and dealing the blocks round-robin measured 4 %
+    // faster in fp16 (2 x 384 x 384, 8 heads, offsets N(0, 24 px) per head: 3.22 -> 3.09 ms for the whole backward),
+    // the same in bf16 and 4 % slower in fp32 (4.23 -> 4.42 ms), which keeps its bands.
+    const unsigned blk = logical_block(blockIdx.x, gridDim.x, A.xcd_swizzle && (A.per_head[0] == 0 || sizeof(T) == 4));
     int khq = (int)(blk * Cfg::HQ_PER_BLOCK + threadIdx.x / LPH);   // (key pixel, head)
     const bool tail = khq >= A.nhq;
     if (tail) khq = A.nhq - 1;
