@@ -69,7 +69,9 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
         for (int e = 0; e < EPV; ++e) { dk[w][e] = 0.f; dv[w][e] = 0.f; }
     }
 
-    const int src = A.per_head[0] ? head : 0;          // whose index lists this head's queries
+    const bool pairs_per_head = A.per_head[0] != 0;    // (also the layout of the pair array: PairLayout)
+    const int src = pairs_per_head ? head : 0;         // whose index lists this head's queries
+    const PairLayout pairs((uint32_t)head, (uint32_t)M, (uint32_t)A.h, pairs_per_head);
     const int *perm = A.perm + (size_t)src * npix;
     const int *centre = A.centre + (size_t)src * npix;
     const int *bin_start = A.bin_start + (size_t)src * A.nrows * A.W;   // start of a bin within its row
@@ -188,9 +190,8 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
                 const int info = (u < step && tf + u < total) ? __builtin_amdgcn_ds_bpermute(from, info_m) : 0;
                 const bool hit = (info >> 12) != 0;
                 const int i_lo = info & 7, i_hi = (info >> 3) & 7, j_lo = (info >> 6) & 7, j_hi = (info >> 9) & 7;
-                const int qhq = qp * A.h + head;
                 if constexpr (ONE) {
-                    const typename PairOf<T>::Word da = ((const typename PairOf<T>::Word *)A.dl_ws)[(size_t)qhq * M + (hit ? j_lo * WN + i_lo : 0)];
+                    const typename PairOf<T>::Word da = ((const typename PairOf<T>::Word *)A.dl_ws)[(size_t)pairs.at((uint32_t)qp, (uint32_t)(hit ? j_lo * WN + i_lo : 0))];
                     float dl_t, a_t;
                     PairOf<T>::unpack(da, dl_t, a_t);
                     bt.dl[u] = hit ? dl_t : 0.f;
@@ -200,7 +201,7 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
                     if (hit) {                          // several taps of one query on this key simply add up
                         for (int j = j_lo; j <= j_hi; ++j)
                             for (int i = i_lo; i <= i_hi; ++i) {
-                                const typename PairOf<T>::Word da = ((const typename PairOf<T>::Word *)A.dl_ws)[(size_t)qhq * M + j * WN + i];
+                                const typename PairOf<T>::Word da = ((const typename PairOf<T>::Word *)A.dl_ws)[(size_t)pairs.at((uint32_t)qp, (uint32_t)(j * WN + i))];
                                 float dl_t, a_t;
                                 PairOf<T>::unpack(da, dl_t, a_t);
                                 bt.dl[u] += dl_t;

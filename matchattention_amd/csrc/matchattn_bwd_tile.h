@@ -40,6 +40,7 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
     const __amdgpu_buffer_rsrc_t rdm = make_rsrc(A.dmo, (uint32_t)A.nhq * 4u);
     const __amdgpu_buffer_rsrc_t rda = make_rsrc(A.d_attn, A.d_attn ? (uint32_t)A.nhq * (uint32_t)(M * 2) : 0u);
     const __amdgpu_buffer_rsrc_t rws = make_rsrc(A.dl_ws, (uint32_t)A.nhq * (uint32_t)(M * 4));   // (dl, a) as two halves per tap
+    const bool pairs_per_head = A.per_head[0] != 0;    // layout of the pair array (PairLayout): the inverse index's flag, not the tile buckets'
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(S.defer, (uint32_t)A.nhq);
     const int sub = threadIdx.x % LPH;
     const int grp = threadIdx.x / LPH;
@@ -52,13 +53,11 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
     const float nscale = -A.scale;
 
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
-    const int nitems = nchunks * nhg;
     const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
     // XCD x takes the x-th share of the work list (consecutive chunks, shares of equal cost: tile_chunks_kernel), the
     // head groups of a chunk being neighbours in the item order; bounds read from scratch memory are clamped
     const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
     const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
-    (void)nitems;
     const bool per_head = *S.per_head != 0;
     // (the order of an item's prologue follows the forward kernel: staging addresses, the two index loads, the
     // staging loads, then the first pass's rows while the staging loads are in flight; the work-list entry is
@@ -88,6 +87,7 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
         const int hgrp = item - (item / nhg) * nhg;
         const int bin = clampi(entry.x, 0, S.nbins - 1), part = max(entry.y, 0);
         const int head = hgrp * HPG + hslot;
+        const PairLayout pairs((uint32_t)head, (uint32_t)M, (uint32_t)A.h, pairs_per_head);
         int lo, hi;
         bucket_bounds(S, per_head ? head : 0, bin, lo, hi);
         const int row = bin / S.bins_per_row, tx = bin - row * S.bins_per_row;
@@ -308,9 +308,8 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
             for (int bb = 0; bb < 4; ++bb) { dw[bb] *= inv[bb]; cd[bb] = c[bb] * dw[bb]; }
             coef9<R>(cd, cd9);
             const bool mine = valid && fits && !far;
-            // (the dead offset leaves room for the tap offsets added below: kDeadOffset + 280 would wrap to a valid one;
-            // the host keeps the scratch array below 0xFFFFF000 bytes)
-            const uint32_t ws_off = (mine && sub == 0) ? (uint32_t)hq * (uint32_t)(M * 4) : 0xFFFFF000u;
+            // (offsets of lanes that store nothing are chosen per store: a dead base plus a tap's offset could wrap into
+            // the array)
 #pragma unroll
             for (int j = 0; j < WN; ++j)
 #pragma unroll
@@ -323,9 +322,10 @@ __global__ __launch_bounds__(kTileNT, 2) void bwd_h16_tile_kernel(BwdArgs A, Til
                         a2[d] = (float)(half_t)(e[j][i + d] * cc);                // the stored attention value
                         g[j][i + d] = dl2[d];
                     }
-                    // (dl, a) pairs of two taps: one 8-byte store
-                    buf_store8(rws, ws_off + (uint32_t)((j * WN + i) * 4),
-                               u32x2{PairOf<T>::pack(dl2[0], a2[0]), PairOf<T>::pack(dl2[1], a2[1])});
+                    // (dl, a) pairs of two taps (neighbours in either layout of the pair array): one 8-byte store
+                    static_assert(WN % 2 == 0 && M % 2 == 0, "two taps of a window row are neighbours in both layouts of the pair array");
+                    const uint32_t off = (mine && sub == 0) ? pairs.at((uint32_t)pix, (uint32_t)(j * WN + i)) * 4u : kDeadOffset;
+                    buf_store8(rws, off, u32x2{PairOf<T>::pack(dl2[0], a2[0]), PairOf<T>::pack(dl2[1], a2[1])});
                 }
             {
                 float dx, dy;

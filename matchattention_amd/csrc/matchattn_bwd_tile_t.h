@@ -34,6 +34,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArg
     const __amdgpu_buffer_rsrc_t rdm = make_rsrc(A.dmo, (uint32_t)A.nhq * (uint32_t)(2 * ES));
     const __amdgpu_buffer_rsrc_t rda = make_rsrc(A.d_attn, A.d_attn ? (uint32_t)A.nhq * (uint32_t)(M * ES) : 0u);
     const __amdgpu_buffer_rsrc_t rws = make_rsrc(A.dl_ws, (uint32_t)A.nhq * (uint32_t)(M * PairOf<T>::kBytes));
+    const bool pairs_per_head = A.per_head[0] != 0;    // layout of the pair array (PairLayout): the inverse index's flag, not the tile buckets'
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(S.defer, (uint32_t)A.nhq);
     const int sub = threadIdx.x % LPH;
     const int grp = threadIdx.x / LPH;
@@ -41,13 +42,11 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArg
     const uint32_t lane_lds = (uint32_t)(hslot * Cfg::HB + sub * 16);
 
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
-    const int nitems = nchunks * nhg;
     const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
     // XCD x takes the x-th share of the work list (consecutive chunks, shares of equal cost: tile_chunks_kernel), the
     // head groups of a chunk being neighbours in the item order; bounds read from scratch memory are clamped
     const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
     const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
-    (void)nitems;
     const bool per_head = *S.per_head != 0;
 #if MA_TILE_QUEUE
     // items are claimed from a counter per XCD, two ahead; the index reaches the workgroup through LDS between
@@ -74,6 +73,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArg
         const int hgrp = item - (item / nhg) * nhg;
         const int bin = clampi(entry.x, 0, S.nbins - 1), part = max(entry.y, 0);
         const int head = hgrp * HPG + hslot;
+        const PairLayout pairs((uint32_t)head, (uint32_t)M, (uint32_t)A.h, pairs_per_head);
         int lo, hi;
         bucket_bounds(S, per_head ? head : 0, bin, lo, hi);
         const int row = bin / S.bins_per_row, tx = bin - row * S.bins_per_row;
@@ -231,17 +231,18 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArg
                     T t2[2] = {Tr::from_f(dx), Tr::from_f(dy)};
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, t2), rdm, wr ? (int)((uint32_t)hq * 4u) : (int)kDeadOffset, 0, 0);
                 }
-                // (a dead offset with room for the whole row: M * 8 bytes added to kDeadOffset would wrap into the
-                // array; the host keeps the array below 0xFFFFF000 bytes)
-                const uint32_t p_off = wr ? (uint32_t)hq * (uint32_t)(M * PairOf<T>::kBytes) : 0xFFFFF000u;
+                // (offsets of lanes that store nothing are chosen per store: a dead base plus a tap's offset could wrap
+                // into the array)
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
 #pragma unroll
                     for (int i = 0; i < WN; ++i)
                     {
                         const auto pw = PairOf<T>::pack(g[j][i], Tr::round(attn_value<R>(shared, lg, st, c9, j, i)));
-                        if constexpr (PairOf<T>::kBytes == 8) buf_store8(rws, p_off + (uint32_t)((j * WN + i) * 8), pw);
-                        else __builtin_amdgcn_raw_buffer_store_b32(pw, rws, (int)(p_off + (uint32_t)((j * WN + i) * 4)), 0, 0);
+                        const uint32_t p_off = wr ? pairs.at((uint32_t)pix, (uint32_t)(j * WN + i)) *
+                                                        (uint32_t)PairOf<T>::kBytes : kDeadOffset;
+                        if constexpr (PairOf<T>::kBytes == 8) buf_store8(rws, p_off, pw);
+                        else __builtin_amdgcn_raw_buffer_store_b32(pw, rws, (int)p_off, 0, 0);
                     }
             }
 

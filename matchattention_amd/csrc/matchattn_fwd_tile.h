@@ -302,7 +302,6 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     // sees one band of neighbouring tiles.  Within that share the workgroups claim items from a counter
     // (MA_TILE_QUEUE; a fixed stride without it).
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
-    const int nitems = nchunks * nhg;
     // Item -> (chunk, head group).  The head groups of a chunk are neighbours in the list: the items an XCD has in
     // flight then cover whole pixel rows of a block of tiles.  (With the head group as the slow index an XCD would
     // touch one 128-byte line in every 128 * nhg bytes, which its L2 maps to a fraction of its sets.)
@@ -312,7 +311,6 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     // (bounds read from scratch memory are clamped before they become indices)
     const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
     const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
-    (void)nitems;
     const bool per_head = *S.per_head != 0;
     // Memory round trips of an item, in order: its work-list entry (fetched one item ahead), the bounds of its
     // bucket, the pixel indices of its first two passes -- issued before the staging loads, which return

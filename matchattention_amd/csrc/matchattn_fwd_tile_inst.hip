@@ -19,11 +19,9 @@ static int launch_tile(const FwdArgs &A, const TileSort &S, hipStream_t s) {
     typedef TileCfg<CH, R, kTileW, kTileH, VPL> Cfg;
     if (A.h % Cfg::HPG != 0) return -1;
     FwdArgs B = A;
-    const int nhg = A.h / Cfg::HPG;
-    (void)nhg;
     launch_tile_chunks(S, A.h, Cfg::QPP, s);
-    // persistent grid: a few workgroups per CU, a multiple of the 8 XCDs
-    const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);   // persistent: two workgroups fit a CU's LDS
+    // persistent grid: a multiple of the 8 XCDs; two workgroups fit a CU's LDS
+    const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);
     timer_mark(false, s);
     hipLaunchKernelGGL((fwd_h16_tile_kernel<CH, R, kTileW, kTileH, VPL>), dim3(grid), dim3(kTileNT), 0, s, B, S);
     timer_mark(true, s);

@@ -96,13 +96,11 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArg
     for (int u = 0; u < VPL; ++u) vec_off[u] = (uint32_t)((u ^ par) * LPH * 16);
 
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
-    const int nitems = nchunks * nhg;
     const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
     // XCD x takes the x-th share of the work list (consecutive chunks, shares of equal cost: tile_chunks_kernel), the
     // head groups of a chunk being neighbours in the item order; bounds read from scratch memory are clamped
     const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
     const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
-    (void)nitems;
     const bool per_head = *S.per_head != 0;
 #if MA_TILE_QUEUE
     // items are claimed from a counter per XCD, two ahead; the index reaches the workgroup through LDS between
