@@ -42,13 +42,17 @@ struct BwdArgs {
 //   an offset per head: [pixel][head][tap], a head-query's taps contiguous (the heads' candidates are unrelated; the
 //   block layout measured 10 % slower there).
 // Both are "pixel base + head term + block * stride + tap % 2"; a lane fixes the head term and the stride once.
+#ifndef MA_PAIR_BLOCK
+#define MA_PAIR_BLOCK 4
+#endif
+constexpr uint32_t kPairBlock = MA_PAIR_BLOCK;     // taps per block: (2r+2)^2 is a multiple of 4
 struct PairLayout {
     uint32_t pix_stride, head_term, stride;
     __device__ __forceinline__ PairLayout(uint32_t head, uint32_t M, uint32_t h, bool per_head)
-        : pix_stride(M * h), head_term(per_head ? head * M : head * 2u), stride(per_head ? 2u : 2u * h) {}
+        : pix_stride(M * h), head_term(per_head ? head * M : head * kPairBlock), stride(per_head ? kPairBlock : kPairBlock * h) {}
     // index (in pairs) of tap m of this lane's head at pixel pix
     __device__ __forceinline__ uint32_t at(uint32_t pix, uint32_t m) const {
-        return pix * pix_stride + head_term + __umul24(m >> 1, stride) + (m & 1u);
+        return pix * pix_stride + head_term + __umul24(m / kPairBlock, stride) + (m % kPairBlock);
     }
 };
 
