@@ -112,7 +112,9 @@ def test_both_backward_modes_agree_with_autograd(hip_lib, mode, dt, offs, clamp,
     ("interior", True, True, 32, 2, (2, 23, 41, 4), True), ("stereo", False, True, 32, 2, (1, 37, 70, 8), True),
     ("mixed", True, False, 32, 1, (2, 23, 41, 4), True), ("mixed", False, False, 64, 2, (1, 19, 50, 2), False),
     ("mixed", True, True, 16, 2, (1, 40, 33, 8), True), ("stereo", True, True, 64, 1, (3, 9, 17, 2), False),
-    ("mixed", True, True, 32, 2, (2, 6, 7, 2), True), ("interior", False, True, 16, 1, (1, 8, 130, 4), True)])
+    ("mixed", True, True, 32, 2, (2, 6, 7, 2), True), ("interior", False, True, 16, 1, (1, 8, 130, 4), True),
+    # three images whose last strip of tiles is 2 wide, one offset per pixel (the blocked layout of the pair array)
+    ("mixed", False, True, 32, 2, (3, 20, 150, 2), True)])
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32, torch.bfloat16], ids=["f16", "f32", "bf16"])
 def test_lds_tile_backward_matches_autograd(hip_lib, dt, offs, per_head, clamp, Ch, r, shape, with_dattn):
     # backward_mode=1: pass A on LDS tiles (bucketed queries; unclamped offsets exercise the flagged finishing run)
@@ -190,7 +192,10 @@ def test_row_skip_does_not_change_results(hip_lib):
     ("stereo", False, True, 32, 2, (1, 37, 70, 8)), ("mixed", True, True, 32, 2, (2, 23, 41, 4)),
     ("mixed", True, False, 32, 1, (2, 23, 41, 4)), ("mixed", False, False, 64, 2, (1, 19, 50, 2)),
     ("stereo", True, True, 64, 1, (3, 9, 17, 2)), ("mixed", True, False, 16, 2, (1, 40, 33, 8)),
-    ("mixed", True, True, 32, 2, (2, 6, 7, 2)), ("interior", False, True, 16, 1, (1, 8, 130, 4))])
+    ("mixed", True, True, 32, 2, (2, 6, 7, 2)), ("interior", False, True, 16, 1, (1, 8, 130, 4)),
+    # one tile row 188 tiles wide; one tile column 313 tiles tall; three images whose last strip of tiles is 2 wide
+    ("stereo", False, True, 16, 2, (1, 6, 3000, 4)), ("mixed", True, True, 32, 2, (1, 2500, 7, 2)),
+    ("mixed", False, True, 32, 2, (3, 20, 150, 2))])
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32, torch.bfloat16], ids=["f16", "f32", "bf16"])
 def test_lds_tile_forward_matches_oracle(hip_lib, dt, offs, per_head, clamp, Ch, r, shape):
     # forward_lds=1: queries bucketed by K/V tile, every tap read from LDS; without the input clamp some
