@@ -37,6 +37,15 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+# HBM bytes per backward call, per kernel, from the same two counters (profiles/bwd_gather_cfg4_cfg2.md)
+MEASURED_BWD_TRAFFIC_BYTES = {
+    ("cfg4_cross", "bwd_tile_f16"): {
+        "bwd_h16_tile_kernel": (2 * 737252 + 606083) * 1024,      # pass A: 2.0 x FETCH_SIZE + WRITE_SIZE (KiB)
+        "bwd_key_kernel": (2 * 545658 + 294912) * 1024,           # pass B
+    },
+}
+
+
 def _events_ms(fn, steps, warmup):
     import torch
     for _ in range(warmup):
@@ -349,7 +358,9 @@ def main():
                           "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall_ms,
                           "higher_is_better": True, "dtype": str(wl.dtype).split(".")[-1], "data": "synthetic",
                           "config": {"workload": wl.name, "kernel": _cabi.last_backward_kernel()},
-                          "algorithmic_GBps": nbytes / (ev_ms * 1e-3) / 1e9, "call_ms_mean": ev_ms, "call_ms_min": ev_min}))
+                          "algorithmic_GBps": nbytes / (ev_ms * 1e-3) / 1e9, "call_ms_mean": ev_ms, "call_ms_min": ev_min,
+                          "algorithmic_bytes_per_call": nbytes,
+                          "traffic": MEASURED_BWD_TRAFFIC_BYTES.get((args.workload, _cabi.last_backward_kernel()))}))
         return
     if args.direct:
         _cabi.set_option("forward_lds", 0)
