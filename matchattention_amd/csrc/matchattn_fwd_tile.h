@@ -548,7 +548,103 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
         int far = !(gmax - imax < kSharedExpLimit);               // needs the exact per-sub-window softmax
         asm volatile("" : "+v"(far));                             // decided here, so that the logits die with the softmax
         half2_t ap[WN][HW];
-        {
+        if constexpr (kMatrixSum) {
+            // Both lanes of a head-query hold all its logits.  Each takes half of the window's rows (lane `sub` rows
+            // sub * HR .. sub * HR + HR - 1) through the exponentials, the row sums and the final products, and the two
+            // exchange the partial sums of the sub-windows and their finished rows of weights with ds_swizzle (lane ^ 16
+            // is the other lane of the pair; the crossbar of the LDS, no memory and no vector ALU cycles): half of the
+            // exponentials and conversions, the most expensive instructions of the softmax, per lane.
+            constexpr int HR = WN / 2;
+            constexpr int kSwapHalves = 0x401f;            // ds_swizzle bit mode: and 0x1f, or 0, xor 0x10
+            auto other_f = [&](float x) __attribute__((always_inline)) {
+                return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), kSwapHalves));
+            };
+            const bool hi_rows = sub != 0;
+            float e[HR][WN];
+            const float gl = gmax * kLog2e;
+#pragma unroll
+            for (int jj = 0; jj < HR; ++jj)
+#pragma unroll
+                for (int i = 0; i < HW; ++i) {
+                    const half2_t l2 = hi_rows ? lgp[jj + HR][i] : lgp[jj][i];
+                    e[jj][2 * i] = __builtin_amdgcn_exp2f((float)l2.x * kLog2e - gl);
+                    e[jj][2 * i + 1] = __builtin_amdgcn_exp2f((float)l2.y * kLog2e - gl);
+                }
+            // row sums over columns 0 .. WN-2 (west sub-windows) and 1 .. WN-1 (east), as subwindow_sum forms them
+            float rl[HR], rr[HR];
+#pragma unroll
+            for (int jj = 0; jj < HR; ++jj) {
+                float inner = e[jj][1];
+#pragma unroll
+                for (int i = 2; i < WN - 1; ++i) inner += e[jj][i];
+                rl[jj] = e[jj][0] + inner;
+                rr[jj] = inner + e[jj][WN - 1];
+            }
+            // The sums over the rows every sub-window holds (1 .. WN-2) are added in subwindow_sum's order,
+            // ((r1 + r2) + r3) + r4 at WN = 6, so that the result has the bits it had when one lane did it all: the lane
+            // of the low rows sends its partial sum r1 + .. + r(HR-1), the lane of the high rows its rows one by one.
+            float send_l[HR], send_r[HR];                  // [0 .. HR-2]: the partial sum, or inner rows; [HR-1]: my edge row
+            {
+                float pl = rl[1], pr = rr[1];
+#pragma unroll
+                for (int t = 2; t < HR; ++t) { pl += rl[t]; pr += rr[t]; }
+#pragma unroll
+                for (int t = 0; t < HR - 1; ++t) {
+                    send_l[t] = hi_rows ? rl[t] : pl;
+                    send_r[t] = hi_rows ? rr[t] : pr;
+                }
+                send_l[HR - 1] = hi_rows ? rl[HR - 1] : rl[0];
+                send_r[HR - 1] = hi_rows ? rr[HR - 1] : rr[0];
+            }
+            float got_l[HR], got_r[HR];
+#pragma unroll
+            for (int t = 0; t < HR; ++t) { got_l[t] = other_f(send_l[t]); got_r[t] = other_f(send_r[t]); }
+            // low lane: partial = mine, the high rows = theirs; high lane: partial = theirs, the high rows = mine
+            float il = hi_rows ? got_l[0] : send_l[0], ir = hi_rows ? got_r[0] : send_r[0];
+#pragma unroll
+            for (int t = 0; t < HR - 1; ++t) {
+                il += hi_rows ? rl[t] : got_l[t];
+                ir += hi_rows ? rr[t] : got_r[t];
+            }
+            float ssum[4], c[4], c9[3][3];
+            ssum[0] = (hi_rows ? got_l[HR - 1] : send_l[HR - 1]) + il;    // north-west: row 0 + rows 1 .. WN-2
+            ssum[1] = (hi_rows ? got_r[HR - 1] : send_r[HR - 1]) + ir;
+            ssum[2] = il + (hi_rows ? send_l[HR - 1] : got_l[HR - 1]);    // south-west: rows 1 .. WN-2 + row WN-1
+            ssum[3] = ir + (hi_rows ? send_r[HR - 1] : got_r[HR - 1]);
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) c[bb] = w[bb] * __builtin_amdgcn_rcpf(ssum[bb]);
+            coef9<R>(c, c9);
+            half2_t mine[HR][HW], theirs[HR][HW];
+#pragma unroll
+            for (int jj = 0; jj < HR; ++jj) {
+                // class of my row jj among the window's rows: first, last, or in between
+                float cr[3];
+#pragma unroll
+                for (int ii = 0; ii < 3; ++ii)
+                    cr[ii] = jj == 0 ? (hi_rows ? c9[1][ii] : c9[0][ii]) : (jj == HR - 1 ? (hi_rows ? c9[2][ii] : c9[1][ii]) : c9[1][ii]);
+#pragma unroll
+                for (int i = 0; i < HW; ++i) {
+                    // product of two floats rounded once to fp16, one instruction per weight (a multiplication and a
+                    // packed conversion round twice, and take three instructions per pair)
+                    uint32_t pr;
+                    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(pr) : "v"(e[jj][2 * i]), "v"(cr[cls<R>(2 * i)]));
+                    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(pr) : "v"(e[jj][2 * i + 1]), "v"(cr[cls<R>(2 * i + 1)]));
+                    mine[jj][i] = as_h2(pr);
+                }
+            }
+#pragma unroll
+            for (int jj = 0; jj < HR; ++jj)
+#pragma unroll
+                for (int i = 0; i < HW; ++i)
+                    theirs[jj][i] = as_h2((uint32_t)__builtin_amdgcn_ds_swizzle((int)h2_as_u32(mine[jj][i]), kSwapHalves));
+#pragma unroll
+            for (int jj = 0; jj < HR; ++jj)
+#pragma unroll
+                for (int i = 0; i < HW; ++i) {
+                    ap[jj][i] = hi_rows ? theirs[jj][i] : mine[jj][i];
+                    ap[jj + HR][i] = hi_rows ? mine[jj][i] : theirs[jj][i];
+                }
+        } else {
             float e[WN][WN];
             const float gl = gmax * kLog2e;
 #pragma unroll
@@ -593,6 +689,11 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
             if (s >= LAST0 && drop_last) return;
 #pragma unroll
             for (int t = 0; t < G; ++t) {
+                // One fused multiply-add per tap and channel, nothing wider: left free to contract across statements the
+                // compiler joins the two taps of one weight pair into a two-element dot product for a single channel of
+                // one vector, which rounds differently -- and which vector of the head a lane holds depends on where the
+                // bucket order puts the query.
+#pragma clang fp contract(on)
                 const int i = i0 + t;
                 const float am = (float)((i & 1) ? ap[j][i >> 1].y : ap[j][i >> 1].x);
 #pragma unroll

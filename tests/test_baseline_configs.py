@@ -79,6 +79,12 @@ def test_large_maps_forward_whole_map(hip_lib, name):
     wl, inp = _inputs(name)
     H, W = inp["H"], inp["W"]
     out, attn = hip_forward(hip_lib, inp["max_offset"], inp["q"], inp["k"], inp["v"], H, W, wl.r, wl.scale)
+    # A second run puts the head-queries into other lanes (the order inside a bucket is first come, first served) and
+    # must give the same bits: with millions of head-queries a single channel rounded differently in one lane position
+    # shows here and nowhere at the sizes of the small cases.
+    out2, attn2 = hip_forward(hip_lib, inp["max_offset"], inp["q"], inp["k"], inp["v"], H, W, wl.r, wl.scale)
+    assert torch.equal(out, out2) and torch.equal(attn, attn2)
+    del out2, attn2
     out, attn = out.cpu(), attn.cpu()
     dt = inp["q"].dtype
     cpu = [inp[n].cpu() for n in ("max_offset", "q", "k", "v")]
