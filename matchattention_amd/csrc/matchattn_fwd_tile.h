@@ -271,7 +271,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(S.defer, (uint32_t)A.nhq);
     // With two lanes per head-query the pair is lanes l and l ^ 16 of a wavefront (not neighbours): the sum of a
     // tap's |q - k| over the pair's 32 channels is then what one matrix instruction delivers to both lanes
-    // (see pair_ones below), and the vector ALU is left with the subtractions and the sign masks.
+    // (see row_ones0 / row_ones1 below), and the vector ALU is left with the subtractions and the sign masks.
     constexpr bool kMatrixSum = LPH == 2 && VPL == 2;
     const int lane_w = threadIdx.x & 63;
     const int sub = kMatrixSum ? ((lane_w >> 4) & 1) : (int)(threadIdx.x % LPH);
@@ -279,12 +279,16 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     const int hslot = grp % HPG, gi = grp / HPG;
     // A operand of v_mfma_f32_16x16x32_f16 (16 x 32, lane i + 16 (k / 8) holds A[i][k..k+7]) that is 1 where row i and
     // column block k / 8 belong to the same half of the wavefront's four 16-lane blocks and 0 elsewhere: with the
-    // |q - k| halves as the B operand (lane j + 16 b holds column j, rows 8 b .. 8 b + 7) every lane receives, in each
-    // of its four result registers, the sum over the 8 halves of lanes l and l ^ 16.
+    // |q - k| halves as the B operand (lane j + 16 b holds column j, rows 8 b .. 8 b + 7) a result row holds the sum
+    // over the 8 halves of lanes l and l ^ 16.  A lane receives rows 4 b .. 4 b + 3 of its column in its four result
+    // registers; row_ones0 has its ones in the rows i % 4 == 0 only, row_ones1 in the rows i % 4 == 1, so that an
+    // accumulator chained through one instruction with each keeps the two sums apart in registers 0 and 1.
     typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
     const uint32_t one_bits = (((lane_w & 15) >= 8) == (lane_w >= 32)) ? 0x3c003c00u : 0u;
-    [[maybe_unused]] const half8_t pair_ones = __builtin_bit_cast(half8_t, u32x4{one_bits, one_bits, one_bits, one_bits});
+    const uint32_t ob0 = (lane_w & 3) == 0 ? one_bits : 0u, ob1 = (lane_w & 3) == 1 ? one_bits : 0u;
+    [[maybe_unused]] const half8_t row_ones0 = __builtin_bit_cast(half8_t, u32x4{ob0, ob0, ob0, ob0});
+    [[maybe_unused]] const half8_t row_ones1 = __builtin_bit_cast(half8_t, u32x4{ob1, ob1, ob1, ob1});
     // Lane `sub` owns the 16-byte vectors sub, sub + LPH, ... of its head, so that the lanes of one LDS read
     // touch adjacent 16-byte pieces (vectors 2 sub, 2 sub + 1 would put them 32 bytes apart: 2-way bank
     // conflicts).  With two vectors per lane, odd lane groups take theirs in the opposite order: one LDS
@@ -482,6 +486,11 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 const int i = i0 + t;
                 float sum;
                 if constexpr (kMatrixSum) {
+                    // The two vectors of a lane go through two matrix instructions that leave their sums in different
+                    // result rows (row_ones0 / row_ones1), and the vector ALU adds the two: which of a head's vectors is a
+                    // lane's vector 0 depends on its lane group (`par`), and one sum chained through both instructions
+                    // would round in that order (seen once in 10^9 taps as a logit one fp16 ulp apart between two runs);
+                    // an addition does not care.
                     f32x4_t acc4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int u = 0; u < VPL; ++u) {
@@ -489,9 +498,10 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             ad[e] = h2_as_u32(as_h2(qv[u][e]) - as_h2(buf[s & 1][t][u][e])) & 0x7fff7fffu;
-                        acc4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(pair_ones, __builtin_bit_cast(half8_t, ad), acc4, 0, 0, 0);
+                        acc4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(u == 0 ? row_ones0 : row_ones1, __builtin_bit_cast(half8_t, ad), acc4, 0, 0, 0);
                     }
-                    sum = acc4[0];
+                    static_assert(!kMatrixSum || VPL == 2, "one result row per vector of a lane");
+                    sum = acc4[0] + acc4[1];
                 } else {
                     sum = l1_sum<T>(qv[0], buf[s & 1][t][0]);
 #pragma unroll
