@@ -185,9 +185,22 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
 #pragma unroll
             for (int i = 0; i < kChunkKeep; ++i) bucket_bounds_at(S, 0, kept_bin[i], tile[i].row(), tile[i].col(), lo[i], hi[i]);
 #pragma unroll
+            for (int i = 0; i < kChunkKeep; ++i) kept_n[i] = hi[i] - lo[i];
+            // the other heads two at a time, their loads for all kept buckets issued together: a memory round trip per
+            // pair of heads (one per head and bucket made this kernel, with eight heads, as long as the sort's own)
+            for (int hd = 1; hd < nh; hd += 2) {
+                const int hd2 = min(hd + 1, nh - 1);
+                int lo2[kChunkKeep], hi2[kChunkKeep];
+#pragma unroll
+                for (int i = 0; i < kChunkKeep; ++i) {
+                    bucket_bounds_at(S, hd, kept_bin[i], tile[i].row(), tile[i].col(), lo[i], hi[i]);
+                    bucket_bounds_at(S, hd2, kept_bin[i], tile[i].row(), tile[i].col(), lo2[i], hi2[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < kChunkKeep; ++i) kept_n[i] = max(kept_n[i], max(hi[i] - lo[i], hi2[i] - lo2[i]));
+            }
+#pragma unroll
             for (int i = 0; i < kChunkKeep; ++i) {
-                kept_n[i] = hi[i] - lo[i];
-                if (nh > 1) kept_n[i] = max(kept_n[i], population(tile[i]));
                 if (b0 + i >= b1) kept_n[i] = 0;
                 price(kept_n[i], sum, cost_sum);
             }
