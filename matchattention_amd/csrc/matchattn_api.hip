@@ -265,7 +265,7 @@ ma::SortArgs sort_args(const void *max_offset, int dtype, int B, int H, int W, i
     ma::SortArgs S;
     S.mo = max_offset; S.dtype = dtype; S.L = B * H * W; S.N = H * W; S.H = H; S.W = W; S.h = h;
     S.bin_shift = bin_shift; S.row_shift = row_shift; S.rows_per_img = sl.rows_per_img; S.force = force; S.centre = nullptr;
-    S.shared_perm = 0;
+    S.shared_perm = 0; S.pop = nullptr;
     S.bins_per_row = sl.bins_per_row; S.nbins = sl.nbins; S.nrows = sl.nrows;
     S.rowtot = (int *)(ws + sl.rowtot_off); S.per_head = (int *)(ws + sl.flag_off); S.count = (int *)(ws + sl.count_off);
     S.rank = (int *)(ws + sl.rank_off); S.perm = (int *)(ws + sl.perm_off);
@@ -374,6 +374,7 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
             char *ws = (char *)workspace;
             ma::SortArgs S = sort_args(max_offset, dtype, B, H, W, h, sl, ws, ma::kTileLog2[0], ma::kTileLog2[1], 1);
             S.shared_perm = 1;
+            S.pop = (int *)(ws + tl.chunk_off);          // (the work list's own array: populations first, chunk starts later)
             launch_sort(S, sl, L, h, ws, false, s, P.shared_offsets);
             if (hipError_t e = hipGetLastError())
                 return fail(MATCHATTN_ERR_LAUNCH, "matchattn_forward_ws: sort launch failed: %s", hipGetErrorString(e));
@@ -728,6 +729,7 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
                 char *tws = ws + bl.tile_off;
                 ma::SortArgs TS = sort_args(max_offset, dtype, B, H, W, h, bl.tl.sl, tws, ma::kTileLog2[0], ma::kTileLog2[1], 1);
                 TS.shared_perm = 1;
+                TS.pop = (int *)(tws + bl.tl.chunk_off);
                 launch_sort(TS, bl.tl.sl, L, h, tws, false, s);
                 const ma::TileSort T = tile_sort_args(TS, bl.tl, tws);
                 switch (dtype) {

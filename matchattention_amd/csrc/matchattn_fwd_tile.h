@@ -150,22 +150,13 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
     const int b0 = min((int)threadIdx.x * per, S.nbins), b1 = min(b0 + per, S.nbins);
     const int nh = *S.per_head ? h : 1;
     const int full_cost = (kTileCap + qpp - 1) / qpp * kPassCost + kChunkFixedCost;
-    auto population = [&](const TileWalk &at) __attribute__((always_inline)) {
-        int n = 0;
-        for (int hd = 0; hd < nh; ++hd) {
-            int lo, hi;
-            bucket_bounds_at(S, hd, at.bin(), at.row(), at.col(), lo, hi);
-            n = max(n, hi - lo);
-        }
-        return n;
-    };
     auto price = [&](int n, int &chunks, int &cost) __attribute__((always_inline)) {
         const int full = n / kTileCap, rem = n - full * kTileCap;
         chunks += full + (rem ? 1 : 0);
         cost += full * full_cost + (rem ? (rem + qpp - 1) / qpp * kPassCost + kChunkFixedCost : 0);
     };
-    // Up to kChunkKeep buckets of a thread stay in registers -- tile and population, the populations of head 0 fetched by
-    // loads that do not depend on one another: one memory round trip instead of one per bucket, and the second walk reads
+    // Up to kChunkKeep buckets of a thread stay in registers -- tile and population, the populations fetched by loads
+    // that do not depend on one another: one memory round trip instead of one per bucket, and the second walk reads
     // nothing.  Larger maps park the populations in chunk_start between the walks.
     constexpr int kChunkKeep = 4;
     const bool keep = per <= kChunkKeep;
@@ -182,22 +173,16 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
                 kept_bin[i] = at.bin();
                 if (i + 1 < per) at.next();               // (uniform; past the thread's last bucket the tile repeats and is masked below)
             }
+            if (nh > 1) {
+                // heads with their own orders: the sort's scatter kernel has left every bucket's largest population
+                // over the heads in chunk_start (one load per bucket here instead of four per bucket and head)
 #pragma unroll
-            for (int i = 0; i < kChunkKeep; ++i) bucket_bounds_at(S, 0, kept_bin[i], tile[i].row(), tile[i].col(), lo[i], hi[i]);
+                for (int i = 0; i < kChunkKeep; ++i) kept_n[i] = clampi(chunk_start[kept_bin[i]], 0, S.L);   // (read from scratch memory: bounded)
+            } else {
 #pragma unroll
-            for (int i = 0; i < kChunkKeep; ++i) kept_n[i] = hi[i] - lo[i];
-            // the other heads two at a time, their loads for all kept buckets issued together: a memory round trip per
-            // pair of heads (one per head and bucket made this kernel, with eight heads, as long as the sort's own)
-            for (int hd = 1; hd < nh; hd += 2) {
-                const int hd2 = min(hd + 1, nh - 1);
-                int lo2[kChunkKeep], hi2[kChunkKeep];
+                for (int i = 0; i < kChunkKeep; ++i) bucket_bounds_at(S, 0, kept_bin[i], tile[i].row(), tile[i].col(), lo[i], hi[i]);
 #pragma unroll
-                for (int i = 0; i < kChunkKeep; ++i) {
-                    bucket_bounds_at(S, hd, kept_bin[i], tile[i].row(), tile[i].col(), lo[i], hi[i]);
-                    bucket_bounds_at(S, hd2, kept_bin[i], tile[i].row(), tile[i].col(), lo2[i], hi2[i]);
-                }
-#pragma unroll
-                for (int i = 0; i < kChunkKeep; ++i) kept_n[i] = max(kept_n[i], max(hi[i] - lo[i], hi2[i] - lo2[i]));
+                for (int i = 0; i < kChunkKeep; ++i) kept_n[i] = hi[i] - lo[i];
             }
 #pragma unroll
             for (int i = 0; i < kChunkKeep; ++i) {
@@ -206,7 +191,14 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
             }
         } else {
             for (int pos = b0; pos < b1; ++pos, at.next()) {
-                const int n = population(at);
+                int n;
+                if (nh > 1) {
+                    n = clampi(chunk_start[at.bin()], 0, S.L);    // (left there by the sort's scatter kernel)
+                } else {
+                    int lo, hi;
+                    bucket_bounds_at(S, 0, at.bin(), at.row(), at.col(), lo, hi);
+                    n = hi - lo;
+                }
                 chunk_start[at.bin()] = n;                // (population for now: the second walk prices the chunks from it)
                 price(n, sum, cost_sum);
             }

@@ -38,6 +38,8 @@ struct SortArgs {
     int *perm;             // [h][L]
     int *centre;           // optional [h][L]: centre of the entry at the same position, (cy << 16) | (cx & 0xffff),
                            //   each saturated to int16 (enough to decide which taps reach a key); or null
+    int *pop;              // optional [nbins]: when the heads have their own orders, the scatter kernel leaves the largest
+                           //   population of each bin over the heads here (the LDS-tile work list is cut from it); or null
     int *per_head;         // the 256-byte flag block (zero on entry, layout below): [kFlagPerHead] heads need their own
                            //     permutation, [kFlagIncoherent] number of (pixel, head) pairs whose target is not next to
                            //     their left neighbour's
@@ -268,6 +270,22 @@ __global__ __launch_bounds__(1024) void sort_rowtot_scan_kernel(SortArgs S) {
 // With S.shared_perm the copies of head 0's order are left out.
 __global__ __launch_bounds__(256) void sort_scatter_kernel(SortArgs S) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;       // head * L + pix
+    // By the way, for the consumer that cuts the bins into chunks (one workgroup, which would otherwise fetch the
+    // bounds of every bin once per head through one CU): the largest population of bin `idx` over the heads.
+    if (S.pop && idx < S.nbins && sort_useful(S) && *S.per_head) {
+        const int row = idx / S.bins_per_row, tx = idx - row * S.bins_per_row;
+        const int row_n = min(row + 1, S.nrows - 1), bin_n = min(idx + 1, S.nbins - 1);
+        int n = 0;
+#pragma unroll 4
+        for (int hd = 0; hd < S.h; ++hd) {
+            const int row_start = S.rowtot[hd * S.nrows + row], next_row = S.rowtot[hd * S.nrows + row_n];
+            const int start = S.count[hd * S.nbins + idx], next = S.count[hd * S.nbins + bin_n];
+            const int lo = clampi(row_start + start, 0, S.L);
+            const int hi = clampi(tx + 1 < S.bins_per_row ? row_start + next : (row + 1 < S.nrows ? next_row : S.L), lo, S.L);
+            n = max(n, hi - lo);
+        }
+        S.pop[idx] = n;
+    }
     if (idx >= S.h * S.L) return;
     const int hd = idx / S.L, pix = idx - hd * S.L;
     if (!sort_useful(S)) {
