@@ -500,6 +500,32 @@ def test_fused_module_forward_is_bit_identical_to_the_separate_steps(hip_lib, dt
     assert rel_err(got_out.cpu(), want_out) <= tol and rel_err(got_attn.cpu(), want_attn) <= tol
 
 
+def test_fused_concat_rows_that_are_not_whole_16_byte_pieces(hip_lib):
+    # one head at r = 2: the concatenated row is C + 36 halves, 8 bytes short of a multiple of 16, so the vector kernels'
+    # 16-byte stores cannot be used and the fused call takes the generic kernel -- same results to the tolerance, not
+    # to the bit, as the separate steps (which write contiguous tensors through the vector kernel)
+    from matchattention_amd import _cabi, fused_module_forward
+    dt, Ch, h, r, (B, H, W) = torch.float16, 32, 1, 2, (2, 21, 30)
+    N, C = H * W, h * Ch
+    g = torch.Generator().manual_seed(8)
+    q, k, v, gate = (torch.randn(B, N, C, generator=g).to(dt).cuda() for _ in range(4))
+    rel = (torch.randn(B, N, 1, 2, generator=g) * 6.0).to(dt).cuda()
+    scale = Ch ** -0.5
+    mo, out, attn, cat = _module_steps(rel, q, k, v, gate, H, W, r, h,
+                                       lambda mo, q, k, v: hip_forward(hip_lib, mo, q, k, v, H, W, r, scale))
+    assert _cabi.last_forward_kernel().startswith("fwd_tiled_f16")
+    got_cat = fused_module_forward(rel, q, k, v, H, W, [r, r], h, scale, gate=gate, concat=True)
+    assert _cabi.last_forward_kernel().startswith("fwd_generic_f16"), _cabi.last_forward_kernel()
+    got_out, got_attn = fused_module_forward(rel, q, k, v, H, W, [r, r], h, scale, gate=gate)     # contiguous outputs
+    assert _cabi.last_forward_kernel().startswith("fwd_tiled_f16")
+    assert torch.equal(got_out, out) and torch.equal(got_attn, attn)
+    assert torch.isfinite(got_cat).all()
+    want_out, want_attn = O.forward(mo.cpu(), q.cpu(), k.cpu(), v.cpu(), H, W, [r, r], scale)
+    want_out = gate.cpu() * want_out
+    assert rel_err(got_cat[..., :C].cpu(), want_out) <= TOL[dt]
+    assert rel_err(got_cat[..., C:].reshape(B, N, h, -1).cpu(), want_attn) <= TOL[dt]
+
+
 def test_fused_forward_accepts_any_row_stride(hip_lib):
     # rows that are not a multiple of 16 bytes leave the vector kernels; results stay the same
     from matchattention_amd import _cabi
