@@ -640,10 +640,14 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
                 for (int i = 0; i < HW; ++i) {
                     // product of two floats rounded once to fp16, one instruction per weight (a multiplication and a
-                    // packed conversion round twice, and take three instructions per pair)
+                    // packed conversion round twice, and take three instructions per pair).  The compiler's hazard
+                    // checks do not look into inline assembly, so the block carries its own wait states: one before an
+                    // instruction that may read the result of the exponential or reciprocal just before it, one
+                    // between the two halves of the register, one before the next reader.
                     uint32_t pr;
-                    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(pr) : "v"(e[jj][2 * i]), "v"(cr[cls<R>(2 * i)]));
-                    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(pr) : "v"(e[jj][2 * i + 1]), "v"(cr[cls<R>(2 * i + 1)]));
+                    asm("s_nop 0\n\tv_fma_mixlo_f16 %0, %1, %2, 0\n\ts_nop 0\n\tv_fma_mixhi_f16 %0, %3, %4, 0\n\ts_nop 0"
+                        : "=&v"(pr)
+                        : "v"(e[jj][2 * i]), "v"(cr[cls<R>(2 * i)]), "v"(e[jj][2 * i + 1]), "v"(cr[cls<R>(2 * i + 1)]));
                     mine[jj][i] = as_h2(pr);
                 }
             }
