@@ -522,11 +522,13 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 } else {
                     typedef float float2_t __attribute__((ext_vector_type(2)));
                     const half2_t l16 = __builtin_convertvector(float2_t{held, sum}, half2_t);
-                    // (float)half * scale in one instruction per half (the compiler's own choice is a conversion and a
-                    // multiplication each)
-                    float f_lo, f_hi;
-                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(f_lo) : "v"(h2_as_u32(l16)), "v"(nscale));
-                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(f_hi) : "v"(h2_as_u32(l16)), "v"(nscale));
+                    // (float)half * scale in one instruction per half: written as a fused multiply-add with a zero addend
+                    // the compiler selects v_fma_mix_f32, which reads the half in place (for a plain product it converts
+                    // first and multiplies then).  Not inline assembly: the compiler's hazard checks do not look into
+                    // it, and its destination may be a register that a matrix instruction still in flight is going to
+                    // write (the unused rows of an earlier tap's result) -- one scheduling strategy put it there.
+                    const float f_lo = __builtin_fmaf((float)l16.x, nscale, 0.0f);
+                    const float f_hi = __builtin_fmaf((float)l16.y, nscale, 0.0f);
                     lgp[j][i >> 1] = __builtin_convertvector(float2_t{f_lo, f_hi}, half2_t);
                     uint32_t pinned = h2_as_u32(lgp[j][i >> 1]);
                     asm volatile("" : "+v"(pinned));
@@ -639,16 +641,13 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                     cr[ii] = jj == 0 ? (hi_rows ? c9[1][ii] : c9[0][ii]) : (jj == HR - 1 ? (hi_rows ? c9[2][ii] : c9[1][ii]) : c9[1][ii]);
 #pragma unroll
                 for (int i = 0; i < HW; ++i) {
-                    // product of two floats rounded once to fp16, one instruction per weight (a multiplication and a
-                    // packed conversion round twice, and take three instructions per pair).  The compiler's hazard
-                    // checks do not look into inline assembly, so the block carries its own wait states: one before an
-                    // instruction that may read the result of the exponential or reciprocal just before it, one
-                    // between the two halves of the register, one before the next reader.
-                    uint32_t pr;
-                    asm("s_nop 0\n\tv_fma_mixlo_f16 %0, %1, %2, 0\n\ts_nop 0\n\tv_fma_mixhi_f16 %0, %3, %4, 0\n\ts_nop 0"
-                        : "=&v"(pr)
-                        : "v"(e[jj][2 * i]), "v"(cr[cls<R>(2 * i)]), "v"(e[jj][2 * i + 1]), "v"(cr[cls<R>(2 * i + 1)]));
-                    mine[jj][i] = as_h2(pr);
+                    // product of two floats rounded once to fp16, one instruction per weight (v_fma_mixlo_f16 /
+                    // v_fma_mixhi_f16, selected for a fused multiply-add with a zero addend; the plain product became a
+                    // multiplication and a packed conversion: two roundings, three instructions per pair)
+                    half2_t t2;
+                    t2.x = (half_t)__builtin_fmaf(e[jj][2 * i], cr[cls<R>(2 * i)], 0.0f);
+                    t2.y = (half_t)__builtin_fmaf(e[jj][2 * i + 1], cr[cls<R>(2 * i + 1)], 0.0f);
+                    mine[jj][i] = t2;
                 }
             }
 #pragma unroll
