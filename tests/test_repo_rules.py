@@ -59,3 +59,17 @@ def test_measured_traffic_tables_name_existing_workloads():
         assert w in WORKLOADS and k.startswith("fwd_") and v > 0
     for (w, k), per_kernel in bench.MEASURED_BWD_TRAFFIC_BYTES.items():
         assert w in WORKLOADS and k.startswith("bwd_") and all(b > 0 for b in per_kernel.values())
+
+
+def test_no_inline_assembly_instructions_in_the_kernel_that_uses_the_matrix_unit():
+    """The compiler's hazard checks do not look into inline assembly, and its destination may be a register that a
+    matrix instruction in flight still writes: the kernels of matchattn_fwd_tile.h (the only ones with matrix
+    instructions) keep to builtins and plain code; empty asm statements that pin a register are fine."""
+    import re
+    src = open(os.path.join(ROOT, "matchattention_amd", "csrc", "matchattn_fwd_tile.h")).read()
+    assert "__builtin_amdgcn_mfma" in src
+    for m in re.finditer(r'asm\s*(?:volatile)?\s*\(\s*"([^"]*)"', src):
+        assert m.group(1).strip() == "", m.group(0)
+    # and the helper it would inherit inline assembly from is not called beside the matrix instructions
+    body = src[src.index("if constexpr (kMatrixSum) {"):]
+    assert "l1_sum" not in body[:body.index("} else {")]
