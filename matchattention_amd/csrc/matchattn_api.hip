@@ -156,11 +156,6 @@ bool bwd_tiled_shape(int CH, int rx, int dtype) {
     return false;
 }
 
-int default_vpl(int CH, int R, int dtype) {
-    (void)CH; (void)R; (void)dtype;
-    return 1;
-}
-
 }  // namespace
 
 extern "C" {
@@ -362,7 +357,7 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
     int rc = -1;
     if (variant != 0 && rx <= 2 && tiled_ok(ptrs, 5, L, C, CH, dtype) &&
         (reinterpret_cast<uintptr_t>(attn) & 7u) == 0 && A.out_row_bytes % 16 == 0 && A.attn_row_bytes % 8 == 0 && small_views) {
-        const int vpl = variant > 0 ? variant : default_vpl(CH, rx, dtype);
+        const int vpl = variant > 0 ? variant : 1;      // vectors per lane of the direct kernels
         // LDS-tile path: bucket the queries by K/V tile, one workgroup per tile and head group, then the
         // generic kernel for the (normally empty) list of queries a tile could not serve
         if (workspace && P.rel_heads == 0 && tile_wanted(O, B, H, W, C, h, rx, ry, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
@@ -651,8 +646,10 @@ bool bwd_gather_possible(const Options &O, int B, int H, int W, int C, int h, in
     if (O.backward_mode == 0 || O.forward_variant == 0 || C % h) return false;
     const int CH = C / h;
     const long long L = (long long)B * H * W;
+    const unsigned long long M = (unsigned long long)(2 * rx + 2) * (2 * rx + 2);
+    // (the pair array is indexed with 32 bits, PairLayout::at: at most 2^32 - 1 (dl, a) pairs)
     return bwd_tiled_shape(CH, rx, dtype) && (CH * elem_size(dtype)) % 16 == 0 && H < 30000 && W < 30000 &&
-           (unsigned long long)L * C * elem_size(dtype) < 0xFFFFFF00ull;
+           (unsigned long long)L * C * elem_size(dtype) < 0xFFFFFF00ull && (unsigned long long)L * h * M < 0xFFFFFF00ull;
 }
 }  // namespace
 

@@ -57,7 +57,7 @@ struct PairLayout {
 };
 
 // The (logit gradient, attention value) pair pass A leaves per head-query and tap for pass B.  fp32 tensors keep two
-// floats; 16-bit tensors keep two halves in one word: the attention value is a 16-bit number by definition, and the
+// floats; fp16 tensors keep two halves in one word: the attention value is a 16-bit number by definition, and the
 // logit gradient, rounded to half precision (11 bits, like every gradient the call returns; saturated at the largest
 // half instead of overflowing), halves what pass A writes and pass B reads through L2 per tap.
 template <typename T> struct PairOf {
@@ -71,6 +71,22 @@ template <typename T> struct PairOf {
         const half2_t h = as_h2(w);
         dl = (float)h.x;
         a = (float)h.y;
+    }
+};
+// bfloat16 tensors keep two bfloat16 values: the logit gradient then has the exponent range of the tensor type (the
+// definition's own backward keeps it in bfloat16), so that gradients of 1e-6 and below -- a mean-reduced loss without
+// loss scaling -- neither lose bits nor vanish as they would as halves.
+template <> struct PairOf<bf16_t> {
+    static constexpr int kBytes = 4;
+    typedef uint32_t Word;
+    static __device__ __forceinline__ Word pack(float dl, float a) {
+        const uint32_t lo = (uint32_t)__builtin_bit_cast(uint16_t, (bf16_t)dl);
+        const uint32_t hi = (uint32_t)__builtin_bit_cast(uint16_t, (bf16_t)a);
+        return lo | (hi << 16);
+    }
+    static __device__ __forceinline__ void unpack(Word w, float &dl, float &a) {
+        dl = as_f32(w << 16);
+        a = as_f32(w & 0xffff0000u);
     }
 };
 template <> struct PairOf<float> {

@@ -67,10 +67,6 @@ constexpr int kTileCap = MA_TILE_CAP;
 #define MA_TILE_GRID_MULT 2
 #endif
 constexpr int kTileGridMult = MA_TILE_GRID_MULT;
-// 1: the workgroups claim their items from a counter per XCD; 0: fixed stride
-#ifndef MA_TILE_QUEUE
-#define MA_TILE_QUEUE 1
-#endif
 
 // [lo, hi) of bucket `bin` (tile row `row` over all images, tile column `tx`) in the bucket order of head `src`,
 // clamped so that values read from scratch memory never become addresses unchecked
@@ -171,7 +167,8 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
             for (int i = 0; i < kChunkKeep; ++i) {
                 tile[i] = at;
                 kept_bin[i] = at.bin();
-                if (i + 1 < per) at.next();               // (uniform; past the thread's last bucket the tile repeats and is masked below)
+                if (b0 + i + 1 < b1) at.next();           // (past the thread's last bucket the tile repeats and is masked below:
+                                                          //  no position beyond the buckets is ever formed)
             }
             if (nh > 1) {
                 // heads with their own orders: the sort's scatter kernel has left every bucket's largest population
@@ -308,15 +305,14 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     // ---- work items: (head group, chunk of at most kTileCap queries per head of one bucket) ----------
     // A fixed grid of persistent workgroups.  Workgroup ids are dealt round-robin to the 8 XCDs; XCD x takes the
     // x-th share of the work list (consecutive chunks, shares of equal cost: tile_chunks_kernel), so that one L2
-    // sees one band of neighbouring tiles.  Within that share the workgroups claim items from a counter
-    // (MA_TILE_QUEUE; a fixed stride without it).
+    // sees one band of neighbouring tiles.  Within that share the workgroups claim items from a counter.
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
     // Item -> (chunk, head group).  The head groups of a chunk are neighbours in the list: the items an XCD has in
     // flight then cover whole pixel rows of a block of tiles.  (With the head group as the slow index an XCD would
     // touch one 128-byte line in every 128 * nhg bytes, which its L2 maps to a fraction of its sets.)
     auto item_chunk = [&](int it) __attribute__((always_inline)) { return it / nhg; };
     auto item_hgrp = [&](int it) __attribute__((always_inline)) { return it - (it / nhg) * nhg; };
-    const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
+    const int xcd = blockIdx.x & 7;
     // (bounds read from scratch memory are clamped before they become indices)
     const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
     const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
@@ -324,31 +320,22 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     // Memory round trips of an item, in order: its work-list entry (fetched one item ahead), the bounds of its
     // bucket, the pixel indices of its first two passes -- issued before the staging loads, which return
     // after them -- and the first pass's offset and q row, issued while the staging loads are in flight.
-#if MA_TILE_QUEUE
     // The workgroups of an XCD claim the items of its share one by one from a counter (the static stride left
     // up to 8 % of the wave slots idle at the end of the kernel: items take two or three passes).  Thread 0
     // claims two items ahead -- the next item's work-list entry is fetched during the current one -- and hands
     // the index to the workgroup through LDS between the two barriers every item has anyway.  Every workgroup
     // sees the same indices, so all of its wavefronts leave the loop together.
-    (void)per_xcd;
     __shared__ int s_claim;
     int *const queue = S.queue + xcd;
     if (threadIdx.x == 0) s_claim = atomicAdd(queue, 2);
     __syncthreads();
     const int item0 = xcd_start + *(volatile int *)&s_claim;
     int item_next = item0 + 1;
-#else
-    const int item0 = xcd_start + (int)(blockIdx.x >> 3);
-#endif
     int2 entry = int2{0, 0};
     if (item0 < item_end) entry = S.chunk_item[item_chunk(item0)];
-#if MA_TILE_QUEUE
     for (int item = item0; item < item_end;) {
     int claim = 0;
     if (threadIdx.x == 0) claim = atomicAdd(queue, 1);
-#else
-    for (int item = item0; item < item_end; item += per_xcd) {
-#endif
     const int hgrp = item_hgrp(item);
     const int bin = clampi(entry.x, 0, S.nbins - 1), part = max(entry.y, 0);
     // this lane group's head and its share of the bucket
@@ -399,11 +386,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
     for (int u = 0; u < VPL; ++u) qv[u] = buf_load16(rq, (uint32_t)pix * row_bytes + chan_bytes + vec_off[u]);
     // the next item's entry, behind every load this prologue waits for one by one
-#if MA_TILE_QUEUE
     const int item_n = min(item_next, item_end - 1);
-#else
-    const int item_n = min(item + per_xcd, item_end - 1);       // (the last item fetches its own entry again)
-#endif
     const int2 entry_n = S.chunk_item[item_chunk(item_n)];
 
     __syncthreads();                                  // every wave is done with the previous tiles
@@ -413,14 +396,10 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
             *(u32x4 *)(smem + dst[c]) = kv[0][c];
             *(u32x4 *)(smem + Cfg::TILE_BYTES + dst[c]) = kv[1][c];
         }
-#if MA_TILE_QUEUE
     if (threadIdx.x == 0) s_claim = claim;
-#endif
 
     __syncthreads();                                  // tiles are in place
-#if MA_TILE_QUEUE
     const int item_nn = xcd_start + *(volatile int *)&s_claim;
-#endif
 
     // Passes.  The loop is bottom-tested: the registers of the next pass are handed over in straight-line
     // code after the stores, so the wait before them covers the loads only, not the stores just issued.
@@ -480,6 +459,12 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
         for (int i = 0; i < HW; ++i) lgp[WN - 1][i] = half2_t{ninf, ninf};   // stays if the row is left out
         fetch(KT{}, std::integral_constant<int, 0>{});
         float held = 0.f;                               // raw sum of the even tap of a pair until its odd tap is done
+        // Running sum of the raw tap sums, for one purpose: a matrix instruction multiplies the |q - k| of all four
+        // 16-lane blocks of a column by 0 or 1, and 0 x inf = NaN -- a non-finite q or k value (or a difference that
+        // overflows fp16) of one head-query would turn the logits of the unrelated head-query in lanes l ^ 32 into NaN
+        // as well.  The sums are >= 0, so the total is finite exactly when every one of them was; head-queries whose
+        // total is not are left to the generic kernel, which keeps such values local to the query that owns them.
+        [[maybe_unused]] float finite_check = 0.f;
         static_for<0, NSR>([&](auto s_tag) __attribute__((always_inline)) {
             constexpr int s = decltype(s_tag)::value, j = s / SPR, i0 = (s % SPR) * G;
             if constexpr (s + 1 < NSR) {
@@ -507,6 +492,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                     }
                     static_assert(!kMatrixSum || VPL == 2, "one result row per vector of a lane");
                     sum = acc4[0] + acc4[1];
+                    finite_check += sum;
                 } else {
                     sum = l1_sum<T>(qv[0], buf[s & 1][t][0]);
 #pragma unroll
@@ -563,6 +549,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
         for (int i = 1; i < HW - 1; ++i) imax = fmaxf(imax, fmaxf((float)min2[i].x, (float)min2[i].y));
         int far = !(gmax - imax < kSharedExpLimit);               // needs the exact per-sub-window softmax
+        if constexpr (kMatrixSum) far |= !(finite_check < __builtin_inff());   // (false for NaN too)
         asm volatile("" : "+v"(far));                             // decided here, so that the logits die with the softmax
         half2_t ap[WN][HW];
         if constexpr (kMatrixSum) {
@@ -774,10 +761,8 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
         valid = slot < hi;
     } while (__builtin_amdgcn_ballot_w64(valid) != 0);          // later passes have larger slots still
     entry = entry_n;
-#if MA_TILE_QUEUE
     item = item_next;
     item_next = item_nn;
-#endif
     }   // items
 }
 

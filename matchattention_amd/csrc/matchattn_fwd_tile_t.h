@@ -96,34 +96,25 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArg
     for (int u = 0; u < VPL; ++u) vec_off[u] = (uint32_t)((u ^ par) * LPH * 16);
 
     const int nchunks = min(max(S.chunk_start[S.nbins], 0), S.chunk_cap);
-    const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
+    const int xcd = blockIdx.x & 7;
     // XCD x takes the x-th share of the work list (consecutive chunks, shares of equal cost: tile_chunks_kernel), the
     // head groups of a chunk being neighbours in the item order; bounds read from scratch memory are clamped
     const int share_lo = clampi(S.xcd_bounds[xcd], 0, nchunks), share_hi = clampi(S.xcd_bounds[xcd + 1], share_lo, nchunks);
     const int xcd_start = share_lo * nhg, item_end = share_hi * nhg;
     const bool per_head = *S.per_head != 0;
-#if MA_TILE_QUEUE
     // items are claimed from a counter per XCD, two ahead; the index reaches the workgroup through LDS between
     // the two barriers of an item (see the fp16 forward kernel)
-    (void)per_xcd;
     __shared__ int s_claim;
     int *const queue = S.queue + xcd;
     if (threadIdx.x == 0) s_claim = atomicAdd(queue, 2);
     __syncthreads();
     const int item0 = xcd_start + *(volatile int *)&s_claim;
     int item_next = item0 + 1;
-#else
-    const int item0 = xcd_start + (int)(blockIdx.x >> 3);
-#endif
     int2 entry = int2{0, 0};
     if (item0 < item_end) entry = S.chunk_item[item0 / nhg];
-#if MA_TILE_QUEUE
     for (int item = item0; item < item_end;) {
     int claim = 0;
     if (threadIdx.x == 0) claim = atomicAdd(queue, 1);
-#else
-    for (int item = item0; item < item_end; item += per_xcd) {
-#endif
     const int hgrp = item - (item / nhg) * nhg;
     const int bin = clampi(entry.x, 0, S.nbins - 1), part = max(entry.y, 0);
     const int head = hgrp * HPG + hslot;
@@ -170,11 +161,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArg
     u32x4 qv[VPL];
 #pragma unroll
     for (int u = 0; u < VPL; ++u) qv[u] = buf_load16(rq, (uint32_t)pix * row_bytes + chan_bytes + vec_off[u]);
-#if MA_TILE_QUEUE
     const int item_n = min(item_next, item_end - 1);
-#else
-    const int item_n = min(item + per_xcd, item_end - 1);       // (the last item fetches its own entry again)
-#endif
     const int2 entry_n = S.chunk_item[item_n / nhg];
 
     __syncthreads();                                  // every wave is done with the previous tiles
@@ -184,13 +171,9 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArg
             *(u32x4 *)(smem + dst[c]) = kv[0][c];
             *(u32x4 *)(smem + Cfg::TILE_BYTES + dst[c]) = kv[1][c];
         }
-#if MA_TILE_QUEUE
     if (threadIdx.x == 0) s_claim = claim;
-#endif
     __syncthreads();                                  // tiles are in place
-#if MA_TILE_QUEUE
     const int item_nn = xcd_start + *(volatile int *)&s_claim;
-#endif
 
     __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): see the fp16 kernel
     bool valid = slot < hi;
@@ -357,10 +340,8 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArg
         valid = slot < hi;
     } while (__builtin_amdgcn_ballot_w64(valid) != 0);
     entry = entry_n;
-#if MA_TILE_QUEUE
     item = item_next;
     item_next = item_nn;
-#endif
     }   // items
 }
 

@@ -75,6 +75,17 @@ def fused_forward(max_offset, q, k, v, output, attn_out, H, W, win_r, attn_num, 
             B, H, W, C, h, int(win_r[0]), int(win_r[1]), float(scale), dt, _stream_ptr(q.device)))
 
 
+# Dispatcher route.  When ``import match_attention`` fails, the reference's operator falls back to
+# ``torch.ops.match_attention.fused_forward`` (models/match_former_ops.py:34-39), which its extension registers with
+# the schema of models/src/match_former_cuda.cpp:46-49.  The same name and schema are defined here (as a fragment: the
+# reference's own file defines ``match_attention::fused_forward_ops`` in that namespace), so that branch lands in
+# this library as well once ``matchattention_amd`` has been imported.
+_DISPATCH_LIB = torch.library.Library("match_attention", "FRAGMENT")
+_DISPATCH_LIB.define("fused_forward(Tensor max_offset, Tensor q, Tensor k, Tensor v, Tensor(a!) output, "
+                     "Tensor(b!) attn_out, int H, int W, int[] win_r, int attn_num, str attn_type, float scale) -> ()")
+_DISPATCH_LIB.impl("fused_forward", fused_forward, "CUDA")
+
+
 @torch.library.custom_op("matchattention_amd::fused_forward_ops", mutates_args={"output", "attn_out"})
 def fused_forward_ops(max_offset: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                       output: torch.Tensor, attn_out: torch.Tensor, H: int, W: int, win_r: List[int],

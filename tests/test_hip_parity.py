@@ -681,6 +681,69 @@ def test_non_finite_offsets_stay_local(hip_lib, dt, lds, bmode):
     assert torch.isfinite(bad_f[0][0, finite_rows]).all() and torch.isfinite(bad_f[1][0, finite_rows]).all()
 
 
+def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib):
+    # The fp16 LDS-tile kernel adds the |q - k| of a lane pair with a matrix instruction whose zero entries multiply the
+    # values of the other head-queries of the wavefront: 0 * inf = NaN.  A non-finite q or k value (or a difference
+    # that overflows fp16: 6e4 - (-6e4)) must only change the queries that own it or whose window reaches it.
+    from matchattention_amd import _cabi
+    B, H, W, h, Ch, r = 1, 40, 50, 4, 32, 2
+    mo, q, k, v = make_case(B, H, W, h, Ch, r, torch.float16, seed=77, offsets="interior", per_head=False)
+    qb, kb = q.clone(), k.clone()
+    q_poison = {5 * W + 7: float("inf"), 17 * W + 30: float("nan"), 30 * W + 12: 6.0e4}
+    k_poison = {9 * W + 40: -float("inf"), 22 * W + 21: float("nan"), 33 * W + 5: -6.0e4}
+    for n, val in q_poison.items():
+        qb[0, n, 3] = val
+        qb[0, n, Ch + 9] = val
+    for n, val in k_poison.items():
+        kb[0, n, 2 * Ch + 1] = val
+    # the query of the 6e4 entry reaches keys that hold -6e4 in the same channel: the difference overflows
+    kb[0, 30 * W + 12, 3] = -6.0e4
+    k_bad = set(k_poison) | {30 * W + 12}
+    ix = torch.floor(mo[0, :, 0, 0].float()).long()
+    iy = torch.floor(mo[0, :, 0, 1].float()).long()
+    touched = torch.zeros(H * W, dtype=torch.bool)
+    touched[list(q_poison)] = True
+    taps = torch.arange(-r, r + 2)
+    xs = (ix[:, None] + taps[None]).clamp(0, W - 1)          # [N, 2r+2]
+    ys = (iy[:, None] + taps[None]).clamp(0, H - 1)
+    for n in k_bad:
+        py, px = divmod(n, W)
+        touched |= (xs == px).any(1) & (ys == py).any(1)
+    assert 0 < int(touched.sum()) < H * W // 4
+    try:
+        _cabi.set_option("forward_lds", 1)
+        good = hip_forward(hip_lib, *_dev(mo, q, k, v), H, W, r, 0.2)
+        assert _cabi.last_forward_kernel().startswith("fwd_tile_f16")
+        bad = hip_forward(hip_lib, *_dev(mo, qb, kb, v), H, W, r, 0.2)
+        _cabi.set_option("forward_lds", 0)
+        direct = hip_forward(hip_lib, *_dev(mo, qb, kb, v), H, W, r, 0.2)
+    finally:
+        _cabi.set_option("forward_lds", -1)
+    keep = ~touched.cuda()
+    for a, b in zip(good, bad):
+        assert torch.isfinite(b[0, keep]).all()
+        assert torch.equal(a[0, keep], b[0, keep])
+    # the queries that own a poisoned value get what the kernels without a matrix unit give them
+    for a, b in zip(bad, direct):
+        own = touched.cuda()
+        assert torch.equal(torch.isfinite(a[0, own]), torch.isfinite(b[0, own]))
+
+
+def test_bf16_backward_keeps_small_gradients(hip_lib):
+    # upstream gradients of 1e-6 (a mean-reduced loss, no loss scaling): the logit gradient between the two passes of
+    # the gather backward must keep bfloat16's exponent range -- as halves these values lose bits or vanish.
+    B, H, W, h, Ch, r = 1, 20, 24, 2, 32, 2
+    M = (2 * r + 2) ** 2
+    dt = torch.bfloat16
+    mo, q, k, v = make_case(B, H, W, h, Ch, r, dt, seed=5, offsets="interior")
+    g = torch.Generator().manual_seed(3)
+    d_out = (torch.randn(B, H * W, h * Ch, generator=g) * 1e-6).to(dt)
+    d_attn = (torch.randn(B, H * W, h, M, generator=g) * 1e-6).to(dt)
+    scale = Ch ** -0.5
+    got = hip_backward(hip_lib, *_dev(mo, q, k, v), H, W, r, scale, d_out.cuda(), d_attn.cuda())
+    check_grads(got, mo, q, k, v, H, W, r, scale, d_out, d_attn, "bwd small gradients")
+
+
 def test_misaligned_tensors_take_the_generic_kernels(hip_lib):
     # views that start one element into an allocation are not 16-byte aligned: no vector kernel may touch them;
     # the results must agree with the aligned call

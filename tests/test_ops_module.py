@@ -45,6 +45,20 @@ def test_reference_import_name_and_native_signature(hip_lib):
     assert rel_err(output.cpu(), want_out) <= 2e-3 and rel_err(attn_out.cpu(), want_attn) <= 2e-3
 
 
+def test_reference_dispatcher_fallback_route(hip_lib):
+    # the reference's `except ImportError` branch: torch.ops.match_attention.fused_forward with the schema of
+    # models/src/match_former_cuda.cpp:46-49 (registered when the package is imported)
+    import matchattention_amd  # noqa: F401
+    B, H, W, h, Ch, r = 1, 9, 10, 2, 16, 1
+    mo, q, k, v = make_case(B, H, W, h, Ch, r, torch.float16, seed=8)
+    want_out, want_attn = O.forward(mo, q, k, v, H, W, [r, r], 0.25)
+    mo, q, k, v = (t.cuda() for t in (mo, q, k, v))
+    output = torch.zeros_like(v)
+    attn_out = q.new_zeros([B, H * W, h, 16])
+    assert torch.ops.match_attention.fused_forward(mo, q, k, v, output, attn_out, H, W, [r, r], 16, "l1_norm", 0.25) is None
+    assert rel_err(output.cpu(), want_out) <= 2e-3 and rel_err(attn_out.cpu(), want_attn) <= 2e-3
+
+
 def test_opaque_op_survives_torch_compile_tracing(hip_lib):
     from matchattention_amd import MF_FusedForwardOps
     B, H, W, h, Ch, r = 1, 8, 8, 2, 8, 1

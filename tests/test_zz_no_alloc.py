@@ -56,9 +56,16 @@ def test_static_scratch_rejects_maps_beyond_its_capacity(hip_lib):
     # 2 x 544 x 960 x 8 heads needs 72 MiB: an error with the sizes in it, and nothing is launched
     B, H, W, h, Ch, r = 2, 544, 960, 8, 32, 2
     assert hip_lib.matchattn_forward_workspace_bytes(B, H, W, h * Ch, h, r, r, _cabi.F16) > hip_lib.matchattn_static_scratch_bytes()
-    one = torch.zeros(16, device="cuda")
-    rc = hip_lib.matchattn_forward_static(one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(), one.data_ptr(),
-                                          one.data_ptr(), B, H, W, h * Ch, h, r, r, 1.0, _cabi.F16, None)
+    # tensors of the sizes the shape states (0.5 GiB each): were the refusal ever lost, the launch would stay inside them
+    N, C, M = H * W, h * Ch, (2 * r + 2) ** 2
+    qkv = torch.zeros(B, N, C, dtype=torch.float16, device="cuda")
+    out = torch.empty_like(qkv)
+    attn = torch.empty(B, N, h, M, dtype=torch.float16, device="cuda")
+    mo = torch.full((B, N, h, 2), float(r), dtype=torch.float16, device="cuda")
+    rc = hip_lib.matchattn_forward_static(mo.data_ptr(), qkv.data_ptr(), qkv.data_ptr(), qkv.data_ptr(), out.data_ptr(),
+                                          attn.data_ptr(), B, H, W, C, h, r, r, 1.0, _cabi.F16,
+                                          torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
     assert rc == 2
     assert b"scratch" in hip_lib.matchattn_last_error()
 
