@@ -197,10 +197,10 @@ int matchattn_set_option(const char *name, int value) {
 
 namespace {
 struct SortLayout { size_t count_off, rowtot_off, rank_off, perm_off, flag_off, total; int nbins, bins_per_row, nrows, rows_per_img; };
-SortLayout sort_layout(int B, int H, int W, int h, int bin_shift = 3, int row_shift = 0) {
+SortLayout sort_layout(int B, int H, int W, int h, int bin_w, int bin_h = 1) {
     SortLayout s;
-    s.bins_per_row = (W + (1 << bin_shift) - 1) >> bin_shift;
-    s.rows_per_img = (H + (1 << row_shift) - 1) >> row_shift;
+    s.bins_per_row = (W + bin_w - 1) / bin_w;
+    s.rows_per_img = (H + bin_h - 1) / bin_h;
     s.nrows = B * s.rows_per_img;
     s.nbins = s.nrows * s.bins_per_row;
     const size_t L = (size_t)B * H * W;
@@ -217,7 +217,7 @@ SortLayout sort_layout(int B, int H, int W, int h, int bin_shift = 3, int row_sh
 struct TileLayout { SortLayout sl; size_t defer_off, chunk_off, item_off, total; int chunk_cap; };
 TileLayout tile_layout(int B, int H, int W, int h) {
     TileLayout t;
-    t.sl = sort_layout(B, H, W, h, ma::kTileLog2[0], ma::kTileLog2[1]);
+    t.sl = sort_layout(B, H, W, h, ma::kTileDims[0], ma::kTileDims[1]);
     t.defer_off = t.sl.total;
     t.chunk_off = t.defer_off + (((size_t)B * H * W * h + 255) & ~(size_t)255);   // one flag byte per head-query
     t.item_off = t.chunk_off + (((size_t)(t.sl.nbins + 1) * 4 + 255) & ~(size_t)255);
@@ -256,10 +256,10 @@ void launch_sort(const ma::SortArgs &S, const SortLayout &sl, long long L, int h
 
 // Sort arguments over a workspace laid out by sort_layout at `ws`.
 ma::SortArgs sort_args(const void *max_offset, int dtype, int B, int H, int W, int h, const SortLayout &sl, char *ws,
-                       int bin_shift, int row_shift, int force) {
+                       int bin_w, int bin_h, int force) {
     ma::SortArgs S;
     S.mo = max_offset; S.dtype = dtype; S.L = B * H * W; S.N = H * W; S.H = H; S.W = W; S.h = h;
-    S.bin_shift = bin_shift; S.row_shift = row_shift; S.rows_per_img = sl.rows_per_img; S.force = force; S.centre = nullptr;
+    S.bin_w = bin_w; S.bin_h = bin_h; S.rows_per_img = sl.rows_per_img; S.force = force; S.centre = nullptr;
     S.shared_perm = 0; S.pop = nullptr;
     S.bins_per_row = sl.bins_per_row; S.nbins = sl.nbins; S.nrows = sl.nrows;
     S.rowtot = (int *)(ws + sl.rowtot_off); S.per_head = (int *)(ws + sl.flag_off); S.count = (int *)(ws + sl.count_off);
@@ -367,7 +367,7 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
                 return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_ws: workspace of %zu bytes needed, %zu given",
                             tl.total, workspace_bytes);
             char *ws = (char *)workspace;
-            ma::SortArgs S = sort_args(max_offset, dtype, B, H, W, h, sl, ws, ma::kTileLog2[0], ma::kTileLog2[1], 1);
+            ma::SortArgs S = sort_args(max_offset, dtype, B, H, W, h, sl, ws, ma::kTileDims[0], ma::kTileDims[1], 1);
             S.shared_perm = 1;
             S.pop = (int *)(ws + tl.chunk_off);          // (the work list's own array: populations first, chunk starts later)
             launch_sort(S, sl, L, h, ws, false, s, P.shared_offsets);
@@ -622,7 +622,7 @@ bool bwd_tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx
 }
 BwdLayout bwd_gather_layout(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
     BwdLayout l;
-    l.sl = sort_layout(B, H, W, h, 0);              // one bin per target pixel
+    l.sl = sort_layout(B, H, W, h, 1);              // one bin per target pixel
     const size_t nhq = (size_t)B * H * W * h, M = (size_t)(2 * rx + 2) * (2 * rx + 2);
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     l.sort_off = 0;
@@ -710,7 +710,7 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
                             bl.total, workspace ? workspace_bytes : (size_t)0);
             char *ws = (char *)workspace;
             const SortLayout &sl = bl.sl;
-            ma::SortArgs S = sort_args(max_offset, dtype, B, H, W, h, sl, ws, 0, 0, 1);
+            ma::SortArgs S = sort_args(max_offset, dtype, B, H, W, h, sl, ws, 1, 1, 1);
             S.centre = (int *)(ws + bl.centre_off);
             launch_sort(S, sl, L, h, ws, true, s);
             if (hipError_t e = hipGetLastError())
@@ -724,7 +724,7 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
                 // pass A on LDS tiles: a second bucketing (by K/V tile), the tile kernel, then the direct kernel
                 // for the head-queries the tile kernel flagged
                 char *tws = ws + bl.tile_off;
-                ma::SortArgs TS = sort_args(max_offset, dtype, B, H, W, h, bl.tl.sl, tws, ma::kTileLog2[0], ma::kTileLog2[1], 1);
+                ma::SortArgs TS = sort_args(max_offset, dtype, B, H, W, h, bl.tl.sl, tws, ma::kTileDims[0], ma::kTileDims[1], 1);
                 TS.shared_perm = 1;
                 TS.pop = (int *)(tws + bl.tl.chunk_off);
                 launch_sort(TS, bl.tl.sl, L, h, tws, false, s);

@@ -18,15 +18,14 @@
 
 namespace ma {
 
-// Tile of key pixels one workgroup serves (powers of two: the sort shifts by their logarithms).
-#ifndef MA_TILE_W_LOG2
-#define MA_TILE_W_LOG2 4
+// Tile of key pixels one workgroup serves.
+#ifndef MA_TILE_W
+#define MA_TILE_W 16
 #endif
-#ifndef MA_TILE_H_LOG2
-#define MA_TILE_H_LOG2 3
+#ifndef MA_TILE_H
+#define MA_TILE_H 8
 #endif
-constexpr int kTileWLog2 = MA_TILE_W_LOG2, kTileHLog2 = MA_TILE_H_LOG2;
-constexpr int kTileW = 1 << kTileWLog2, kTileH = 1 << kTileHLog2;
+constexpr int kTileW = MA_TILE_W, kTileH = MA_TILE_H;
 
 // Threads per workgroup and the waves per SIMD the register allocation aims for: two workgroups
 // fit a CU's LDS: 8 waves per CU, 2 per SIMD.

@@ -4,7 +4,7 @@
 
 namespace ma {
 
-const int kTileLog2[2] = {kTileWLog2, kTileHLog2};
+const int kTileDims[2] = {kTileW, kTileH};
 const int kTileCapHost = kTileCap;
 void launch_tile_chunks(const TileSort &S, int h, int queries_per_pass, hipStream_t s) {
     hipLaunchKernelGGL(tile_chunks_kernel<0>, dim3(1), dim3(1024), 0, s, S, h, S.chunk_start, queries_per_pass > 0 ? queries_per_pass : 64);

@@ -43,7 +43,7 @@ unsigned tile_grid(unsigned per_cu);
 // consuming kernel takes from a chunk at a time (prices a chunk for the split of the list among the XCDs).  Defined once, beside the fp16 forward tile kernel:
 // a second copy in another translation unit would be a second device kernel of the same name.
 void launch_tile_chunks(const TileSort &S, int h, int queries_per_pass, hipStream_t s);
-extern const int kTileLog2[2];       // log2 of the tile width and height the kernel was built for
+extern const int kTileDims[2];       // tile width and height (key pixels) the kernels were built for
 extern const int kTileCapHost;       // queries per head in one work item of that kernel
 
 int launch_bwd_tiled_f32(const BwdArgs &A, int CH, int R, hipStream_t s, const char **name);

@@ -23,13 +23,13 @@ struct SortArgs {
     const void *mo;
     int dtype;             // MATCHATTN_F32 / F16 / BF16 numbering
     int L, N, H, W, h;     // L = B*N pixels
-    int bin_shift;         // a bin is 2^bin_shift columns wide (3: ordering for locality; 0: exact inverse index)
+    int bin_w;             // a bin is bin_w columns wide (1: exact inverse index; the tile width for the tile buckets)
     int force;             // 1: always sort (inverse index for the backward); 0: only when the probe finds it useful
-    int row_shift;         // a bin is 2^row_shift rows tall (0 except for the tile buckets of the LDS forward)
+    int bin_h;             // a bin is bin_h rows tall (1 except for the tile buckets of the LDS-tile kernels)
     int shared_perm;       // 1: when the heads share head 0's order only perm[0] is written (the consumer reads
                            //    per_head[0] and follows head 0's row); 0: every head's row is always complete
-    int rows_per_img;      // ceil(H / 2^row_shift)
-    int bins_per_row;      // ceil(W / 2^bin_shift)
+    int rows_per_img;      // ceil(H / bin_h)
+    int bins_per_row;      // ceil(W / bin_w)
     int nbins;             // nrows * bins_per_row
     int nrows;             // B * rows_per_img rows of bins
     int *count;            // [h][nbins]  (zero on entry; after the scans: start of the bin within its row)
@@ -89,7 +89,11 @@ __device__ __forceinline__ int pack_centre(float x, float y) {
 __device__ __forceinline__ uint32_t target_cell(const SortArgs &S, float x, float y) {
     const int ix = clampi((int)floorf(fminf(fmaxf(x, -1e6f), 1e6f)), 0, S.W - 1);
     const int iy = clampi((int)floorf(fminf(fmaxf(y, -1e6f), 1e6f)), 0, S.H - 1);
-    return ((uint32_t)(iy >> S.row_shift) << 16) | (uint32_t)(ix >> S.bin_shift);
+    // (unsigned division by a small run-time constant; powers of two take the shift)
+    const uint32_t bw = (uint32_t)S.bin_w, bh = (uint32_t)S.bin_h;
+    const uint32_t cx = (bw & (bw - 1)) == 0 ? (uint32_t)ix >> __builtin_ctz(bw) : (uint32_t)ix / bw;
+    const uint32_t cy = (bh & (bh - 1)) == 0 ? (uint32_t)iy >> __builtin_ctz(bh) : (uint32_t)iy / bh;
+    return (cy << 16) | cx;
 }
 
 __device__ __forceinline__ int target_bin(const SortArgs &S, int pix, float x, float y) {
@@ -160,7 +164,7 @@ __global__ __launch_bounds__(256) void sort_probe_kernel(SortArgs S) {
             // that otherwise bounds this kernel)
             const bool unequal = other[u] && !(x[u] == x0[u] && y[u] == y0[u]);
             if (__builtin_amdgcn_ballot_w64(unequal) != 0 && unequal)
-                differ = differ || (S.bin_shift == 0 ? pack_centre(x[u], y[u]) != pack_centre(x0[u], y0[u])
+                differ = differ || (S.bin_w == 1 ? pack_centre(x[u], y[u]) != pack_centre(x0[u], y0[u])
                                                      : target_cell(S, x[u], y[u]) != target_cell(S, x0[u], y0[u]));
             if (!S.force) n += __builtin_popcountll(__builtin_amdgcn_ballot_w64(incoherent));
         }

@@ -56,6 +56,17 @@ WORKLOADS = {
 }
 
 
+# The operator calls of one MatchStereo-T frame at 1536 x 1536 (reference models/match_stereo.py:13-15,24 and
+# models/convformer.py:353: four levels at 1/32 .. 1/4 of the padded input, both views in the batch, 4 heads), each as
+# the cross-attention call (one position shared by the heads, attention gradient present) and the self-attention call
+# (a position per head).  The fields are spatially smooth, as a model's are.
+MODEL_SHAPES = {
+    f"tiny1536_{hw}x{hw}_c{c}_r{r}_{kind}": Workload(f"tiny1536_{hw}x{hw}_c{c}_r{r}_{kind}", torch.float16, 2, hw, hw, c, 4, r,
+                                                    f"stereo:{hw // 4}" if kind == "cross" else "gauss:2", kind == "self", True)
+    for hw, c, r in ((48, 160, 2), (96, 128, 2), (192, 64, 1), (384, 32, 1)) for kind in ("cross", "self")
+}
+
+
 def clamp_max_offset(max_offset: torch.Tensor, H: int, W: int, r: int) -> torch.Tensor:
     """The clamp the attention module applies before calling the operator
     (reference models/attention_blocks.py:45-59); bounds are rounded to the tensor dtype."""
@@ -73,7 +84,9 @@ def make_inputs(wl: Workload, device="cuda", seed: Optional[int] = None, smooth:
     """Returns dict(max_offset, q, k, v, d_out, d_attn) on `device`, seeded.
     `rows` limits the map to its first rows (a bounded sample of the same workload)."""
     H = wl.H if rows is None else min(rows, wl.H)
-    g = torch.Generator(device=device).manual_seed(1000 + (list(WORKLOADS).index(wl.name) if seed is None else seed))
+    if seed is None:
+        seed = list(WORKLOADS).index(wl.name) if wl.name in WORKLOADS else 100 + list(MODEL_SHAPES).index(wl.name)
+    g = torch.Generator(device=device).manual_seed(1000 + seed)
     N = H * wl.W
 
     def randn(*shape):

@@ -722,7 +722,11 @@ def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib):
     keep = ~touched.cuda()
     for a, b in zip(good, bad):
         assert torch.isfinite(b[0, keep]).all()
-        assert torch.equal(a[0, keep], b[0, keep])
+        # Head-queries that shared a matrix instruction with a poisoned one are recomputed by the generic kernel: the
+        # same values to the operator's tolerance, not necessarily to the bit; all others are untouched.
+        assert rel_err(b[0, keep].float().cpu(), a[0, keep].float().cpu()) <= 2e-3
+        same = (a[0, keep] == b[0, keep]).flatten(1).all(1).float().mean().item()
+        assert same >= 0.95, same
     # the queries that own a poisoned value get what the kernels without a matrix unit give them
     for a, b in zip(bad, direct):
         own = touched.cuda()
