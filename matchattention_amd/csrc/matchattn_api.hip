@@ -197,9 +197,9 @@ int matchattn_set_option(const char *name, int value) {
 
 namespace {
 struct SortLayout { size_t count_off, rowtot_off, rank_off, perm_off, flag_off, total; int nbins, bins_per_row, nrows, rows_per_img; };
-SortLayout sort_layout(int B, int H, int W, int h, int bin_w, int bin_h = 1) {
+SortLayout sort_layout(int B, int H, int W, int h, int bin_w, int bin_h = 1, int sub_h = 1) {
     SortLayout s;
-    s.bins_per_row = (W + bin_w - 1) / bin_w;
+    s.bins_per_row = (W + bin_w - 1) / bin_w * sub_h;
     s.rows_per_img = (H + bin_h - 1) / bin_h;
     s.nrows = B * s.rows_per_img;
     s.nbins = s.nrows * s.bins_per_row;
@@ -217,12 +217,13 @@ SortLayout sort_layout(int B, int H, int W, int h, int bin_w, int bin_h = 1) {
 struct TileLayout { SortLayout sl; size_t defer_off, chunk_off, item_off, total; int chunk_cap; };
 TileLayout tile_layout(int B, int H, int W, int h) {
     TileLayout t;
-    t.sl = sort_layout(B, H, W, h, ma::kTileDims[0], ma::kTileDims[1]);
+    t.sl = sort_layout(B, H, W, h, ma::kTileDims[0], ma::kTileDims[1], ma::kTileDims[1]);
     t.defer_off = t.sl.total;
     t.chunk_off = t.defer_off + (((size_t)B * H * W * h + 255) & ~(size_t)255);   // one flag byte per head-query
-    t.item_off = t.chunk_off + (((size_t)(t.sl.nbins + 1) * 4 + 255) & ~(size_t)255);
+    const int ntiles = t.sl.nbins / ma::kTileDims[1];
+    t.item_off = t.chunk_off + (((size_t)(ntiles + 1) * 4 + 255) & ~(size_t)255);
     // a bucket has ceil(max over heads of its population / cap) chunks: at most nbins + h * L / cap in all
-    t.chunk_cap = (int)std::min<size_t>((size_t)t.sl.nbins + (size_t)B * H * W * h / ma::kTileCapHost + 1, (size_t)1 << 30);
+    t.chunk_cap = (int)std::min<size_t>((size_t)ntiles + (size_t)B * H * W * h / ma::kTileCapHost + 1, (size_t)1 << 30);
     t.total = t.item_off + (((size_t)t.chunk_cap * 8 + 255) & ~(size_t)255);
     return t;
 }
@@ -259,7 +260,7 @@ ma::SortArgs sort_args(const void *max_offset, int dtype, int B, int H, int W, i
                        int bin_w, int bin_h, int force) {
     ma::SortArgs S;
     S.mo = max_offset; S.dtype = dtype; S.L = B * H * W; S.N = H * W; S.H = H; S.W = W; S.h = h;
-    S.bin_w = bin_w; S.bin_h = bin_h; S.rows_per_img = sl.rows_per_img; S.force = force; S.centre = nullptr;
+    S.bin_w = bin_w; S.bin_h = bin_h; S.sub_h = sl.bins_per_row / ((W + bin_w - 1) / bin_w); S.rows_per_img = sl.rows_per_img; S.force = force; S.centre = nullptr;
     S.shared_perm = 0; S.pop = nullptr;
     S.bins_per_row = sl.bins_per_row; S.nbins = sl.nbins; S.nrows = sl.nrows;
     S.rowtot = (int *)(ws + sl.rowtot_off); S.per_head = (int *)(ws + sl.flag_off); S.count = (int *)(ws + sl.count_off);
@@ -275,7 +276,8 @@ ma::TileSort tile_sort_args(const ma::SortArgs &S, const TileLayout &tl, char *w
     T.chunk_item = (int2 *)(ws + tl.item_off); T.chunk_cap = tl.chunk_cap;
     T.queue = S.per_head + ma::kFlagQueue;             // inside the 256-byte flag block the sort zeroes
     T.xcd_bounds = S.per_head + ma::kFlagXcdBounds;
-    T.bins_per_row = tl.sl.bins_per_row; T.nbins = tl.sl.nbins; T.nrows = tl.sl.nrows; T.rows_per_img = tl.sl.rows_per_img;
+    T.sub = S.sub_h;
+    T.bins_per_row = tl.sl.bins_per_row / T.sub; T.nbins = tl.sl.nbins / T.sub; T.nrows = tl.sl.nrows; T.rows_per_img = tl.sl.rows_per_img;
     T.L = S.L;
     return T;
 }

@@ -55,7 +55,8 @@ struct TileSort {
     int *chunk_start;      // [nbins + 1] chunks of the buckets before each one, and their total
     int2 *chunk_item;      // [chunk_cap] work list: (bucket, index of the chunk within it)
     int chunk_cap;
-    int bins_per_row, nbins, nrows, rows_per_img, L;
+    int bins_per_row, nbins, nrows, rows_per_img, L;     // in tiles
+    int sub;               // `count` holds `sub` entries per tile (sub-buckets by the window's row in the tile), tile-major
     int *queue;            // [8] zero on entry: next unclaimed item of each XCD's share of the work list
     int *xcd_bounds;       // [9] chunks [xcd_bounds[x], xcd_bounds[x + 1]) of the work list are XCD x's share (equal cost)
 };

@@ -66,6 +66,10 @@ constexpr int kTileCap = MA_TILE_CAP;
 #define MA_TILE_GRID_MULT 2
 #endif
 constexpr int kTileGridMult = MA_TILE_GRID_MULT;
+// 1: the fp16 forward with 32 channels per head aggregates on the matrix unit (fwd_h16_tile_kernel, V phase)
+#ifndef MA_TILE_MFMA_AGG
+#define MA_TILE_MFMA_AGG 1
+#endif
 
 // [lo, hi) of bucket `bin` (tile row `row` over all images, tile column `tx`) in the bucket order of head `src`,
 // clamped so that values read from scratch memory never become addresses unchecked
@@ -73,8 +77,8 @@ __device__ __forceinline__ void bucket_bounds_at(const TileSort &S, int src, int
     // four independent loads (both candidates for the end are fetched, then one is chosen): one latency
     const int row_start = S.rowtot[src * S.nrows + row];
     const int next_row = S.rowtot[src * S.nrows + min(row + 1, S.nrows - 1)];
-    const int start = S.count[src * S.nbins + bin];
-    const int next = S.count[src * S.nbins + min(bin + 1, S.nbins - 1)];
+    const int start = S.count[(src * S.nbins + bin) * S.sub];
+    const int next = S.count[(src * S.nbins + min(bin + 1, S.nbins - 1)) * S.sub];
     lo = row_start + start;
     hi = tx + 1 < S.bins_per_row ? row_start + next : (row + 1 < S.nrows ? next_row : S.L);
     lo = clampi(lo, 0, S.L);
@@ -256,7 +260,23 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     constexpr int GB = Cfg::GB, HPG = Cfg::HPG, CPP = Cfg::CPP, PSTR = Cfg::PSTR, LPH = Cfg::LPH, QPP = Cfg::QPP;
     constexpr int G = St::G, SPR = St::SPR, NSR = WN * SPR, LAST0 = (WN - 1) * SPR;
 
-    __shared__ __attribute__((aligned(16))) char smem[2 * Cfg::TILE_BYTES];   // K tile, then V tile
+    // With two lanes per head-query and two heads per group (32 channels per head) the aggregation runs on the matrix
+    // unit as well (see the V phase below); it needs 32 - BW pixels of readable zeros behind the V tile and, per
+    // wavefront, one row of weights (24 halves) for each of its 32 head-queries.
+    constexpr bool kMatrixAgg = MA_TILE_MFMA_AGG && LPH == 2 && VPL == 2 && HPG == 2 && CH == 32 && BW <= 24;
+    // The V rectangle then has a pixel stride of 136 bytes: one transposing read touches 8 bytes in each of four 16-byte
+    // pieces of 16 pixels, which a stride of 128 bytes (32 banks) puts on the same banks eight times over and a stride of
+    // 34 banks spreads over all of them (two to three accesses per bank; 128 accesses of two banks on 64 banks).
+    constexpr int VSTR = kMatrixAgg ? PSTR + 8 : PSTR;
+    constexpr int V_OFF = Cfg::TILE_BYTES;
+    constexpr int V_RECT_BYTES = BW * BH * VSTR;
+    constexpr int V_BYTES = kMatrixAgg ? (BW * BH + 32 - BW) * VSTR : Cfg::TILE_BYTES;     // with the zeros behind the rectangle
+    constexpr int V_ZERO16 = (V_OFF + V_RECT_BYTES + 15) / 16 * 16;                         // 16 aligned bytes of those zeros
+    constexpr int WM_ROW_BYTES = 48, WM_WAVE_BYTES = 32 * WM_ROW_BYTES, WM_BYTES = kMatrixAgg ? (kTileNT / 64) * WM_WAVE_BYTES : 0;
+    constexpr int WM_OFF = (V_OFF + V_BYTES + 15) / 16 * 16;
+    static_assert(WM_OFF + WM_BYTES + 64 <= 80 * 1024, "two workgroups per CU");
+    static_assert(!kMatrixAgg || V_ZERO16 + 16 <= V_OFF + V_BYTES, "zeros for the lanes beyond a row");
+    __shared__ __attribute__((aligned(16))) char smem[WM_OFF + WM_BYTES];   // K tile, V tile (+ zeros), weight rows
 
     const int nhg = A.h / HPG;
     const int npix = S.L;
@@ -327,6 +347,9 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     __shared__ int s_claim;
     int *const queue = S.queue + xcd;
     if (threadIdx.x == 0) s_claim = atomicAdd(queue, 2);
+    if constexpr (kMatrixAgg) {                        // the zeros behind the V tile (never written again)
+        for (int i = V_RECT_BYTES + threadIdx.x * 8; i < V_BYTES; i += kTileNT * 8) *(u32x2 *)(smem + V_OFF + i) = u32x2{0, 0};
+    }
     __syncthreads();
     const int item0 = xcd_start + *(volatile int *)&s_claim;
     int item_next = item0 + 1;
@@ -393,7 +416,13 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     for (int c = 0; c < Cfg::CPT; ++c)
         if (dst[c] != 0xffffffffu) {
             *(u32x4 *)(smem + dst[c]) = kv[0][c];
-            *(u32x4 *)(smem + Cfg::TILE_BYTES + dst[c]) = kv[1][c];
+            if constexpr (kMatrixAgg) {                 // (pixel stride VSTR: 8-byte aligned pieces)
+                const uint32_t dv = V_OFF + dst[c] + (dst[c] / PSTR) * (VSTR - PSTR);
+                *(u32x2 *)(smem + dv) = u32x2{kv[1][c][0], kv[1][c][1]};
+                *(u32x2 *)(smem + dv + 8) = u32x2{kv[1][c][2], kv[1][c][3]};
+            } else {
+                *(u32x4 *)(smem + Cfg::TILE_BYTES + dst[c]) = kv[1][c];
+            }
         }
     if (threadIdx.x == 0) s_claim = claim;
 
@@ -671,86 +700,235 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                     ap[j][i].y = (half_t)(e[j][2 * i + 1] * c9[cls<R>(j)][cls<R>(2 * i + 1)]);
                 }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        {   // the first V stage waits for the last attention weight (keeps it below the softmax)
-            uint32_t last = h2_as_u32(ap[WN - 2][HW - 1]);
-            asm volatile("" : "+v"(last));
-            ap[WN - 2][HW - 1] = as_h2(last);
-        }
-        fetch(VT{}, std::integral_constant<int, 0>{});
-
-        // ---- aggregation -----------------------------------------------------------------------
-        float acc[VPL][8];
+        auto store_attn = [&](bool mine) __attribute__((always_inline)) {
+            // The attention row of a head-query (M/2 dwords) leaves in 16-byte pieces dealt to the LPH lanes of the
+            // head-query -- piece p from lane p % LPH -- so that one store instruction covers LPH * 16 contiguous bytes per
+            // head-query (8-byte stores from one lane made nine requests to L2 per row, three quarters of all the
+            // requests of the kernel).  The dwords left over (2 at M = 36) follow as one 8-byte store.
+            {
+                constexpr int NDW = M / 2, NP = NDW / 4, REM = NDW - NP * 4;
+                uint32_t dw[NDW];
 #pragma unroll
-        for (int u = 0; u < VPL; ++u)
+                for (int m = 0; m < NDW; ++m) dw[m] = h2_as_u32(ap[m / HW][m % HW]);
+                const uint32_t a_row = mine ? (uint32_t)pix * A.attn_row_bytes + (uint32_t)head * (uint32_t)(M * 2) : kDeadOffset;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[u][e] = 0.f;
-        static_for<0, NSR>([&](auto s_tag) __attribute__((always_inline)) {
-            constexpr int s = decltype(s_tag)::value, j = s / SPR, i0 = (s % SPR) * G;
-            if constexpr (s + 1 < NSR) {
-                if (s + 1 < LAST0 || !drop_last) fetch(VT{}, std::integral_constant<int, s + 1>{});
-            }
-            if (s >= LAST0 && drop_last) return;
+                for (int t = 0; t * LPH < NP; ++t) {
+                    u32x4 piece = u32x4{dw[0], dw[1], dw[2], dw[3]};
 #pragma unroll
-            for (int t = 0; t < G; ++t) {
-                // One fused multiply-add per tap and channel, nothing wider: left free to contract across statements the
-                // compiler joins the two taps of one weight pair into a two-element dot product for a single channel of
-                // one vector, which rounds differently -- and which vector of the head a lane holds depends on where the
-                // bucket order puts the query.
-#pragma clang fp contract(on)
-                const int i = i0 + t;
-                const float am = (float)((i & 1) ? ap[j][i >> 1].y : ap[j][i >> 1].x);
-#pragma unroll
-                for (int u = 0; u < VPL; ++u)
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[u][e] += am * vec_elem<T>(buf[s & 1][t][u], e);
-            }
-            // this stage's sums are complete before the next stage's reads are issued
-#pragma unroll
-            for (int u = 0; u < VPL; ++u)
-                asm volatile("" : "+v"(acc[u][0]), "+v"(acc[u][1]), "+v"(acc[u][2]), "+v"(acc[u][3]), "+v"(acc[u][4]), "+v"(acc[u][5]), "+v"(acc[u][6]), "+v"(acc[u][7]));
-            __builtin_amdgcn_sched_barrier(0);
-        });
-
-        // ---- stores; what this tile cannot serve is flagged for the generic kernel --------------------
-        // (a flag per head-query, written with the results: no atomics, no zero-fill, and nothing the next
-        // pass has to wait for)
-        const bool mine = valid && fits && !far;
-        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(mine ? 0 : 1), rd, (valid && sub == 0) ? hq : (int)kDeadOffset, 0, 0);
-        u32x4 ov[VPL];
-#pragma unroll
-        for (int u = 0; u < VPL; ++u) ov[u] = vec_pack<T>(acc[u]);
-        if (A.gate) {
-#pragma unroll
-            for (int u = 0; u < VPL; ++u) ov[u] = vec_mul<T>(ov[u], gatev[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < VPL; ++u)
-            buf_store16(ro, mine ? (uint32_t)pix * A.out_row_bytes + chan_bytes + vec_off[u] : kDeadOffset, ov[u]);
-        // The attention row of a head-query (M/2 dwords) leaves in 16-byte pieces dealt to the LPH lanes of the
-        // head-query -- piece p from lane p % LPH -- so that one store instruction covers LPH * 16 contiguous bytes per
-        // head-query (8-byte stores from one lane made nine requests to L2 per row, three quarters of all the
-        // requests of the kernel).  The dwords left over (2 at M = 36) follow as one 8-byte store.
-        {
-            constexpr int NDW = M / 2, NP = NDW / 4, REM = NDW - NP * 4;
-            uint32_t dw[NDW];
-#pragma unroll
-            for (int m = 0; m < NDW; ++m) dw[m] = h2_as_u32(ap[m / HW][m % HW]);
-            const uint32_t a_row = mine ? (uint32_t)pix * A.attn_row_bytes + (uint32_t)head * (uint32_t)(M * 2) : kDeadOffset;
-#pragma unroll
-            for (int t = 0; t * LPH < NP; ++t) {
-                u32x4 piece = u32x4{dw[0], dw[1], dw[2], dw[3]};
-#pragma unroll
-                for (int sl = 0; sl < LPH; ++sl) {
-                    const int pc = t * LPH + sl;
-                    if (pc < NP && sub == sl) piece = u32x4{dw[4 * pc], dw[4 * pc + 1], dw[4 * pc + 2], dw[4 * pc + 3]};
+                    for (int sl = 0; sl < LPH; ++sl) {
+                        const int pc = t * LPH + sl;
+                        if (pc < NP && sub == sl) piece = u32x4{dw[4 * pc], dw[4 * pc + 1], dw[4 * pc + 2], dw[4 * pc + 3]};
+                    }
+                    const int mine_pc = t * LPH + sub;
+                    buf_store16(ra, (mine && mine_pc < NP) ? a_row + (uint32_t)mine_pc * 16u : kDeadOffset, piece);
                 }
-                const int mine_pc = t * LPH + sub;
-                buf_store16(ra, (mine && mine_pc < NP) ? a_row + (uint32_t)mine_pc * 16u : kDeadOffset, piece);
+                static_assert(REM == 0 || REM == 2, "attention rows are a whole number of 8-byte pieces");
+                if (REM == 2)
+                    buf_store8(ra, (mine && sub == NP % LPH) ? a_row + (uint32_t)NP * 16u : kDeadOffset, u32x2{dw[NP * 4], dw[NP * 4 + 1]});
             }
-            static_assert(REM == 0 || REM == 2, "attention rows are a whole number of 8-byte pieces");
-            if (REM == 2)
-                buf_store8(ra, (mine && sub == NP % LPH) ? a_row + (uint32_t)NP * 16u : kDeadOffset, u32x2{dw[NP * 4], dw[NP * 4 + 1]});
+        };
+        if constexpr (kMatrixAgg) {
+            // ---- aggregation on the matrix unit ------------------------------------------------------------------
+            // out^T = V^T W per head: 16 channels x 32 pixels of one row of the staged V rectangle (A operand) times the
+            // weights that 16 head-queries of that head give those 32 pixels (B operand: zero except where the row crosses
+            // a head-query's window), accumulated over the rows the wavefront's windows reach.  The rectangle stays
+            // pixel-major: the A operand comes from ds_read_b64_tr_b16, which hands lane l of a 16-lane block the element
+            // l % 4 of what lanes l / 4 + 4 e (e = 0..3) of the block address -- source lane 4 e + q reads channels
+            // 8 q + 4 cb .. + 3 of pixel e, so lane l = 4 q + c receives channel 8 q + 4 cb + c of four consecutive
+            // pixels.  The B operand goes through LDS: every head-query writes the weights of its window row at its
+            // window's columns into its row of a 24-entry table (zeroed once per pass: a head-query always writes the
+            // same entries), and lane j + 16 g reads entries 8 g .. 8 g + 7 of head-query j.  Result rows 4 b + r of the
+            // two channel blocks are channels 8 b + r and 8 b + 4 + r: lane j + 16 b ends with 16 contiguous bytes of
+            // head-query j's output.  The buckets are ordered by the window's row in the tile, so the 16 queries of a
+            // wavefront start in neighbouring rows: the rows are walked from the first window's first row, a lane whose
+            // window starts `delta` rows later takes its weights from row t - delta.  (Every delta the tile allows is
+            // handled here: which queries share a wavefront depends on the arrival order inside a bucket, and a result
+            // must not.)
+            typedef short short4_t __attribute__((ext_vector_type(4)));
+            typedef short short8_t __attribute__((ext_vector_type(8)));
+            constexpr int kMaxDelta = BH - WN, NT = WN + kMaxDelta;
+            const int grp_local = (lane_w & 15) + ((lane_w >> 5) << 4);       // own head-query within the wavefront
+            const int qq = grp_local >> 1;                                      // its query (0..15); hslot is its head
+            const int cxv = fits ? cx : 0, cyv = fits ? cy : 0;
+            uint32_t cy_mask = 0;
+#pragma unroll
+            for (int c = 0; c <= BH - WN; ++c) cy_mask |= __builtin_amdgcn_ballot_w64(cyv == c) != 0 ? (1u << c) : 0u;
+            const int cy_min = __builtin_ctz(cy_mask), spread = 31 - __builtin_clz(cy_mask) - cy_min;
+            const int delta = cyv - cy_min;
+            const int t_hi = min(spread, kMaxDelta) + WN - 1 - (drop_last ? 1 : 0);     // last row step with a weight in it
+            const bool mine = valid && fits && !far;
+            store_attn(mine);
+            char *const wm = smem + WM_OFF + (threadIdx.x >> 6) * WM_WAVE_BYTES;
+            const int jcol = lane_w & 15, gblk = lane_w >> 4;
+            // lane `sub` of a head-query writes the halves sub, 2 + sub, ... of a window row: kept in the low halves
+            uint32_t wv[WN][HW];
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int i = 0; i < HW; ++i) wv[j][i] = sub ? h2_as_u32(ap[j][i]) >> 16 : h2_as_u32(ap[j][i]);
+            const uint32_t wm_write = (uint32_t)((hslot * 16 + qq) * WM_ROW_BYTES + (cxv + sub) * 2);
+            // (pixels 24 .. 31 of a step lie beyond the rectangle's row: those lanes read zeros, behind the V rectangle)
+            uint32_t wm_read[HPG];
+#pragma unroll
+            for (int hg = 0; hg < HPG; ++hg)
+                wm_read[hg] = gblk < 3 ? (uint32_t)(WM_OFF + (threadIdx.x >> 6) * WM_WAVE_BYTES + (hg * 16 + jcol) * WM_ROW_BYTES + gblk * 16)
+                                       : (uint32_t)V_ZERO16;
+            // source address of the transposing reads: pixel 8 g + e of the first row, channels 8 q .. of head 0, block 0
+            const uint32_t a_base = (uint32_t)(V_OFF + (cy_min * BW + 8 * gblk + ((lane_w & 15) >> 2)) * VSTR + (lane_w & 3) * 16);
+            // owner lanes of the head-queries this lane stores (column jcol of either head), for their pixel and flags
+            int pix_o[HPG], mine_o[HPG], valid_o[HPG];
+#pragma unroll
+            for (int hg = 0; hg < HPG; ++hg) {
+                const int gl = 2 * jcol + hg, owner = (gl & 15) + ((gl >> 4) << 5);
+                pix_o[hg] = __builtin_amdgcn_ds_bpermute(owner * 4, pix);
+                const int fl = __builtin_amdgcn_ds_bpermute(owner * 4, (mine ? 1 : 0) | (valid ? 2 : 0));
+                mine_o[hg] = fl & 1;
+                valid_o[hg] = fl & 2;
+            }
+            u32x4 gate_o[HPG];
+#pragma unroll
+            for (int hg = 0; hg < HPG; ++hg)
+                gate_o[hg] = buf_load16(rgate, (uint32_t)pix_o[hg] * row_bytes + (uint32_t)((hgrp * HPG + hg) * CH * 2 + gblk * 16));
+            f32x4_t dacc[HPG][2];
+#pragma unroll
+            for (int hg = 0; hg < HPG; ++hg)
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) dacc[hg][cb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            *(u32x4 *)(wm + lane_w * 16) = u32x4{0, 0, 0, 0};
+            if (lane_w < (WM_WAVE_BYTES - 1024) / 16) *(u32x4 *)(wm + 1024 + lane_w * 16) = u32x4{0, 0, 0, 0};
+            // One row step's operands: the transposing reads of the V rectangle, this lane's weights for the row into the
+            // table, the reads of the table.  LDS instructions of a wavefront execute in order, so the table may be
+            // rewritten for the next step as soon as the reads of this one are issued: the steps are issued one ahead of
+            // the matrix instructions that use them.
+            struct RowOps { half8_t a[HPG][2], b[HPG]; };
+            RowOps ops[2];
+            auto load_row = [&](auto t_tag) __attribute__((always_inline)) {
+                constexpr int t = decltype(t_tag)::value;
+                RowOps &o = ops[t & 1];
+#pragma unroll
+                for (int hg = 0; hg < HPG; ++hg)
+#pragma unroll
+                    for (int cb = 0; cb < 2; ++cb) {
+                        const short4_t lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) short4_t *)(smem + a_base + (uint32_t)(t * BW * VSTR + hg * CH * 2 + cb * 8)));
+                        const short4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) short4_t *)(smem + a_base + (uint32_t)(t * BW * VSTR + hg * CH * 2 + cb * 8 + 4 * VSTR)));
+                        o.a[hg][cb] = __builtin_bit_cast(half8_t, (short8_t)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+                    }
+#pragma unroll
+                for (int i = 0; i < HW; ++i) {
+                    uint32_t d = 0u;                    // this lane's window row t - delta, if there is one
+#pragma unroll
+                    for (int dl = 0; dl <= kMaxDelta; ++dl)
+                        if (t - dl >= 0 && t - dl < WN) d = delta == dl ? wv[t - dl][i] : d;
+                    *(uint16_t *)(wm + wm_write + 4 * i) = (uint16_t)d;
+                }
+#pragma unroll
+                for (int hg = 0; hg < HPG; ++hg) o.b[hg] = __builtin_bit_cast(half8_t, *(const u32x4 *)(smem + wm_read[hg]));
+            };
+            auto mma_row = [&](auto t_tag) __attribute__((always_inline)) {
+                const RowOps &o = ops[decltype(t_tag)::value & 1];
+#pragma unroll
+                for (int hg = 0; hg < HPG; ++hg)
+#pragma unroll
+                    for (int cb = 0; cb < 2; ++cb)
+                        dacc[hg][cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.a[hg][cb], o.b[hg], dacc[hg][cb], 0, 0, 0);
+            };
+            load_row(std::integral_constant<int, 0>{});
+            static_for<0, NT>([&](auto t_tag) __attribute__((always_inline)) {
+                constexpr int t = decltype(t_tag)::value;
+                if (t > t_hi) return;                  // (the same in every lane)
+                if constexpr (t + 1 < NT) {
+                    if (t + 1 <= t_hi) load_row(std::integral_constant<int, t + 1>{});
+                }
+                mma_row(t_tag);
+            });
+            // A non-finite value in the rectangle multiplies every head-query's zeros: head-queries whose result is not
+            // finite are left to the generic kernel, which keeps such values with the windows that hold them.
+            u32x4 ov[HPG];
+            bool ok_o[HPG];
+            const unsigned long long col = 0x0001000100010001ull << jcol;     // the four lanes that hold column jcol
+#pragma unroll
+            for (int hg = 0; hg < HPG; ++hg) {
+                float o8[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { o8[e] = dacc[hg][0][e]; o8[4 + e] = dacc[hg][1][e]; }
+                ov[hg] = vec_pack<T>(o8);
+                uint32_t any = 0u;                     // bit 15 / 31 set where a half has all exponent bits set
+#pragma unroll
+                for (int e = 0; e < 4; ++e) any |= (ov[hg][e] & 0x7fff7fffu) + 0x04000400u;
+                const unsigned long long bad_m = __builtin_amdgcn_ballot_w64((any & 0x80008000u) != 0u);
+                ok_o[hg] = mine_o[hg] != 0 && (bad_m & col) == 0;
+            }
+            if (A.gate) {
+#pragma unroll
+                for (int hg = 0; hg < HPG; ++hg) ov[hg] = vec_mul<T>(ov[hg], gate_o[hg]);
+            }
+#pragma unroll
+            for (int hg = 0; hg < HPG; ++hg) {
+                const int head_o = hgrp * HPG + hg;
+                // the flag of the head-query (its valid owner wrote nothing: one store per head-query, from block 0's lane)
+                __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(ok_o[hg] ? 0 : 1), rd, (valid_o[hg] && gblk == 0) ? pix_o[hg] * A.h + head_o : (int)kDeadOffset, 0, 0);
+                buf_store16(ro, ok_o[hg] ? (uint32_t)pix_o[hg] * A.out_row_bytes + (uint32_t)(head_o * CH * 2 + gblk * 16) : kDeadOffset, ov[hg]);
+            }
+        } else {
+            __builtin_amdgcn_sched_barrier(0);
+            {   // the first V stage waits for the last attention weight (keeps it below the softmax)
+                uint32_t last = h2_as_u32(ap[WN - 2][HW - 1]);
+                asm volatile("" : "+v"(last));
+                ap[WN - 2][HW - 1] = as_h2(last);
+            }
+            fetch(VT{}, std::integral_constant<int, 0>{});
+
+            // ---- aggregation -----------------------------------------------------------------------
+            float acc[VPL][8];
+    #pragma unroll
+            for (int u = 0; u < VPL; ++u)
+    #pragma unroll
+                for (int e = 0; e < 8; ++e) acc[u][e] = 0.f;
+            static_for<0, NSR>([&](auto s_tag) __attribute__((always_inline)) {
+                constexpr int s = decltype(s_tag)::value, j = s / SPR, i0 = (s % SPR) * G;
+                if constexpr (s + 1 < NSR) {
+                    if (s + 1 < LAST0 || !drop_last) fetch(VT{}, std::integral_constant<int, s + 1>{});
+                }
+                if (s >= LAST0 && drop_last) return;
+    #pragma unroll
+                for (int t = 0; t < G; ++t) {
+                    // One fused multiply-add per tap and channel, nothing wider: left free to contract across statements the
+                    // compiler joins the two taps of one weight pair into a two-element dot product for a single channel of
+                    // one vector, which rounds differently -- and which vector of the head a lane holds depends on where the
+                    // bucket order puts the query.
+    #pragma clang fp contract(on)
+                    const int i = i0 + t;
+                    const float am = (float)((i & 1) ? ap[j][i >> 1].y : ap[j][i >> 1].x);
+    #pragma unroll
+                    for (int u = 0; u < VPL; ++u)
+    #pragma unroll
+                        for (int e = 0; e < 8; ++e) acc[u][e] += am * vec_elem<T>(buf[s & 1][t][u], e);
+                }
+                // this stage's sums are complete before the next stage's reads are issued
+    #pragma unroll
+                for (int u = 0; u < VPL; ++u)
+                    asm volatile("" : "+v"(acc[u][0]), "+v"(acc[u][1]), "+v"(acc[u][2]), "+v"(acc[u][3]), "+v"(acc[u][4]), "+v"(acc[u][5]), "+v"(acc[u][6]), "+v"(acc[u][7]));
+                __builtin_amdgcn_sched_barrier(0);
+            });
+
+            // ---- stores; what this tile cannot serve is flagged for the generic kernel --------------------
+            // (a flag per head-query, written with the results: no atomics, no zero-fill, and nothing the next
+            // pass has to wait for)
+            const bool mine = valid && fits && !far;
+            __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(mine ? 0 : 1), rd, (valid && sub == 0) ? hq : (int)kDeadOffset, 0, 0);
+            u32x4 ov[VPL];
+    #pragma unroll
+            for (int u = 0; u < VPL; ++u) ov[u] = vec_pack<T>(acc[u]);
+            if (A.gate) {
+    #pragma unroll
+                for (int u = 0; u < VPL; ++u) ov[u] = vec_mul<T>(ov[u], gatev[u]);
+            }
+    #pragma unroll
+            for (int u = 0; u < VPL; ++u)
+                buf_store16(ro, mine ? (uint32_t)pix * A.out_row_bytes + chan_bytes + vec_off[u] : kDeadOffset, ov[u]);
+            store_attn(mine);
         }
 
         slot += QPP;

@@ -26,10 +26,13 @@ struct SortArgs {
     int bin_w;             // a bin is bin_w columns wide (1: exact inverse index; the tile width for the tile buckets)
     int force;             // 1: always sort (inverse index for the backward); 0: only when the probe finds it useful
     int bin_h;             // a bin is bin_h rows tall (1 except for the tile buckets of the LDS-tile kernels)
+    int sub_h;             // 1, or bin_h: every bin is cut into bin_h sub-bins by the row inside it, numbered one after the
+                           //   other (bins_per_row, nbins, count then refer to sub-bins): a tile's queries come out ordered
+                           //   by the row of their window in the tile, and its bucket is still one run of the order
     int shared_perm;       // 1: when the heads share head 0's order only perm[0] is written (the consumer reads
                            //    per_head[0] and follows head 0's row); 0: every head's row is always complete
     int rows_per_img;      // ceil(H / bin_h)
-    int bins_per_row;      // ceil(W / bin_w)
+    int bins_per_row;      // ceil(W / bin_w) * sub_h
     int nbins;             // nrows * bins_per_row
     int nrows;             // B * rows_per_img rows of bins
     int *count;            // [h][nbins]  (zero on entry; after the scans: start of the bin within its row)
@@ -93,6 +96,7 @@ __device__ __forceinline__ uint32_t target_cell(const SortArgs &S, float x, floa
     const uint32_t bw = (uint32_t)S.bin_w, bh = (uint32_t)S.bin_h;
     const uint32_t cx = (bw & (bw - 1)) == 0 ? (uint32_t)ix >> __builtin_ctz(bw) : (uint32_t)ix / bw;
     const uint32_t cy = (bh & (bh - 1)) == 0 ? (uint32_t)iy >> __builtin_ctz(bh) : (uint32_t)iy / bh;
+    if (S.sub_h > 1) return (cy << 16) | (cx * (uint32_t)S.sub_h + ((uint32_t)iy - cy * bh));
     return (cy << 16) | cx;
 }
 
@@ -276,16 +280,19 @@ __global__ __launch_bounds__(256) void sort_scatter_kernel(SortArgs S) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;       // head * L + pix
     // By the way, for the consumer that cuts the bins into chunks (one workgroup, which would otherwise fetch the
     // bounds of every bin once per head through one CU): the largest population of bin `idx` over the heads.
-    if (S.pop && idx < S.nbins && sort_useful(S) && *S.per_head) {
-        const int row = idx / S.bins_per_row, tx = idx - row * S.bins_per_row;
-        const int row_n = min(row + 1, S.nrows - 1), bin_n = min(idx + 1, S.nbins - 1);
+    // (per whole bin: the sub_h sub-bins of a tile together)
+    if (S.pop && idx < S.nbins / S.sub_h && sort_useful(S) && *S.per_head) {
+        const int tiles_per_row = S.bins_per_row / S.sub_h;
+        const int row = idx / tiles_per_row, tx = idx - row * tiles_per_row;
+        const int row_n = min(row + 1, S.nrows - 1);
+        const int first = row * S.bins_per_row + tx * S.sub_h, first_n = min(first + S.sub_h, S.nbins - 1);
         int n = 0;
 #pragma unroll 4
         for (int hd = 0; hd < S.h; ++hd) {
             const int row_start = S.rowtot[hd * S.nrows + row], next_row = S.rowtot[hd * S.nrows + row_n];
-            const int start = S.count[hd * S.nbins + idx], next = S.count[hd * S.nbins + bin_n];
+            const int start = S.count[hd * S.nbins + first], next = S.count[hd * S.nbins + first_n];
             const int lo = clampi(row_start + start, 0, S.L);
-            const int hi = clampi(tx + 1 < S.bins_per_row ? row_start + next : (row + 1 < S.nrows ? next_row : S.L), lo, S.L);
+            const int hi = clampi(tx + 1 < tiles_per_row ? row_start + next : (row + 1 < S.nrows ? next_row : S.L), lo, S.L);
             n = max(n, hi - lo);
         }
         S.pop[idx] = n;
