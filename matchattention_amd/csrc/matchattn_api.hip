@@ -215,12 +215,16 @@ SortLayout sort_layout(int B, int H, int W, int h, int bin_w, int bin_h = 1, int
 }
 // LDS-tile forward: buckets of the tile sort, then one flag byte per head-query (left for the generic kernel).
 struct TileLayout { SortLayout sl; size_t defer_off, chunk_off, item_off, total; int chunk_cap; };
-TileLayout tile_layout(int B, int H, int W, int h) {
+// `by_row`: the buckets are ordered by the window's row inside the tile (one sub-bucket per row), which the fp16
+// forward with 32 channels per head wants: its aggregation walks the rows the 16 queries of a wavefront reach.
+bool tile_rows_wanted(int C, int h, int dtype) { return dtype == MATCHATTN_F16 && C / h == 32; }
+TileLayout tile_layout(int B, int H, int W, int h, bool by_row) {
     TileLayout t;
-    t.sl = sort_layout(B, H, W, h, ma::kTileDims[0], ma::kTileDims[1], ma::kTileDims[1]);
+    const int sub = by_row ? ma::kTileDims[1] : 1;
+    t.sl = sort_layout(B, H, W, h, ma::kTileDims[0], ma::kTileDims[1], sub);
     t.defer_off = t.sl.total;
     t.chunk_off = t.defer_off + (((size_t)B * H * W * h + 255) & ~(size_t)255);   // one flag byte per head-query
-    const int ntiles = t.sl.nbins / ma::kTileDims[1];
+    const int ntiles = t.sl.nbins / sub;
     t.item_off = t.chunk_off + (((size_t)(ntiles + 1) * 4 + 255) & ~(size_t)255);
     // a bucket has ceil(max over heads of its population / cap) chunks: at most nbins + h * L / cap in all
     t.chunk_cap = (int)std::min<size_t>((size_t)ntiles + (size_t)B * H * W * h / ma::kTileCapHost + 1, (size_t)1 << 30);
@@ -243,7 +247,7 @@ void launch_sort(const ma::SortArgs &S, const SortLayout &sl, long long L, int h
         else if (S.dtype == MATCHATTN_F16) hipLaunchKernelGGL(ma::sort_probe_kernel<1>, pg, dim3(256), 0, s, S);
         else hipLaunchKernelGGL(ma::sort_probe_kernel<2>, pg, dim3(256), 0, s, S);
     }
-    hipLaunchKernelGGL(ma::sort_count_kernel, dim3((unsigned)((L + 255) / 256), (unsigned)(shared_known ? 1 : h)),
+    hipLaunchKernelGGL(ma::sort_count_kernel, dim3((unsigned)((L + 256 * ma::kCountPerThread - 1) / (256 * ma::kCountPerThread)), (unsigned)(shared_known ? 1 : h)),
                        dim3(256), 0, s, S);
     hipLaunchKernelGGL(ma::sort_rowscan_kernel, dim3((unsigned)sl.nrows, (unsigned)h), dim3(64), 0, s, S);
     hipLaunchKernelGGL(ma::sort_rowtot_scan_kernel, dim3((unsigned)h), dim3(1024), 0, s, S);
@@ -307,7 +311,7 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
 namespace {
 size_t forward_workspace_bytes(const Options &O, int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
     if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || h <= 0) return 0;
-    return tile_wanted(O, B, H, W, C, h, rx, ry, dtype) ? tile_layout(B, H, W, h).total : 0;
+    return tile_wanted(O, B, H, W, C, h, rx, ry, dtype) ? tile_layout(B, H, W, h, tile_rows_wanted(C, h, dtype)).total : 0;
 }
 }  // namespace
 
@@ -363,7 +367,7 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
         // LDS-tile path: bucket the queries by K/V tile, one workgroup per tile and head group, then the
         // generic kernel for the (normally empty) list of queries a tile could not serve
         if (workspace && P.rel_heads == 0 && tile_wanted(O, B, H, W, C, h, rx, ry, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
-            const TileLayout tl = tile_layout(B, H, W, h);
+            const TileLayout tl = tile_layout(B, H, W, h, tile_rows_wanted(C, h, dtype));
             const SortLayout &sl = tl.sl;
             if (workspace_bytes < tl.total)
                 return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_ws: workspace of %zu bytes needed, %zu given",
@@ -524,7 +528,7 @@ int matchattn_forward_deferred(const void *workspace, size_t workspace_bytes,
     if (!count) return fail(MATCHATTN_ERR_ARG, "matchattn_forward_deferred: null count pointer");
     *count = -1;
     if (!workspace || !tile_wanted(options_now(), B, H, W, C, h, rx, ry, dtype)) return MATCHATTN_OK;
-    const TileLayout tl = tile_layout(B, H, W, h);
+    const TileLayout tl = tile_layout(B, H, W, h, tile_rows_wanted(C, h, dtype));
     if (workspace_bytes < tl.total)
         return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_deferred: workspace of %zu bytes needed, %zu given",
                     tl.total, workspace_bytes);
@@ -634,7 +638,7 @@ BwdLayout bwd_gather_layout(const Options &O, int B, int H, int W, int C, int h,
     l.total = l.tile_off;
     l.tile = bwd_tile_wanted(O, B, H, W, C, h, rx, dtype);
     if (l.tile) {
-        l.tl = tile_layout(B, H, W, h);
+        l.tl = tile_layout(B, H, W, h, false);
         l.total += up(l.tl.total);
     }
     return l;

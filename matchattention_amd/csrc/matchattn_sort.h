@@ -190,42 +190,48 @@ __global__ __launch_bounds__(256) void sort_probe_kernel(SortArgs S) {
     }
 }
 
-// Bin counts and ranks.  A workgroup first counts its 256 entries in an LDS table keyed by the low bits of
+// Bin counts and ranks.  A workgroup first counts its entries in an LDS table keyed by the low bits of
 // the bin (neighbouring pixels mostly share a handful of bins), then adds each occupied table entry to
 // the global counter once; an entry whose table slot is taken by another bin goes to the global counter
 // directly.  Ranks inside a bin are arbitrary, as with one atomic per entry, but far fewer contend.
-constexpr int kCountTable = 512;
-__device__ __forceinline__ void count_block(const SortArgs &S, int *count, int *rank_out, bool active, int bin) {
+constexpr int kCountTable = 2048, kCountPerThread = 4;
+// One workgroup counts 1024 pixels of one head, four per thread (grid.y = heads; the rows of heads 1.. exit when the
+// heads share their offsets: head 0 then stands for all of them).  The more entries a workgroup sees, the more of
+// them share a bin: with the sub-buckets of the tile sort 256 entries hardly ever did, and every one of them cost a
+// global atomic.
+__global__ __launch_bounds__(256) void sort_count_kernel(SortArgs S) {
     __shared__ int tag[kCountTable], cnt[kCountTable], base[kCountTable];
+    const int hd = blockIdx.y;
+    if (!sort_useful(S) || (hd > 0 && *S.per_head == 0)) return;    // uniform over the workgroup
     for (int i = threadIdx.x; i < kCountTable; i += blockDim.x) { tag[i] = -1; cnt[i] = 0; }
+    int *const count = S.count + (size_t)hd * S.nbins;
+    int *const rank = S.rank + (size_t)hd * S.L;
+    int pix[kCountPerThread], bin[kCountPerThread], local[kCountPerThread];
+    float x[kCountPerThread], y[kCountPerThread];
+#pragma unroll
+    for (int u = 0; u < kCountPerThread; ++u) {
+        pix[u] = (blockIdx.x * kCountPerThread + u) * (int)blockDim.x + (int)threadIdx.x;
+        load_xy(S.mo, S.dtype, (size_t)min(pix[u], S.L - 1) * S.h + hd, x[u], y[u]);
+    }
     __syncthreads();
-    const int idx = bin & (kCountTable - 1);
-    int local = -1;
-    if (active) {
-        const int old = atomicCAS(&tag[idx], -1, bin);
-        if (old == -1 || old == bin) local = atomicAdd(&cnt[idx], 1);
+#pragma unroll
+    for (int u = 0; u < kCountPerThread; ++u) {
+        local[u] = -1;
+        bin[u] = 0;
+        if (pix[u] < S.L) {
+            bin[u] = target_bin(S, pix[u], x[u], y[u]);
+            const int idx = bin[u] & (kCountTable - 1);
+            const int old = atomicCAS(&tag[idx], -1, bin[u]);
+            if (old == -1 || old == bin[u]) local[u] = atomicAdd(&cnt[idx], 1);
+        }
     }
     __syncthreads();
     for (int i = threadIdx.x; i < kCountTable; i += blockDim.x)
         if (tag[i] >= 0) base[i] = atomicAdd(&count[tag[i]], cnt[i]);
     __syncthreads();
-    if (active) *rank_out = local >= 0 ? base[idx] + local : atomicAdd(&count[bin], 1);
-}
-
-// One workgroup counts 256 pixels of one head (grid.y = heads; the rows of heads 1.. exit when the heads share
-// their offsets: head 0 then stands for all of them).
-__global__ __launch_bounds__(256) void sort_count_kernel(SortArgs S) {
-    const int hd = blockIdx.y;
-    if (!sort_useful(S) || (hd > 0 && *S.per_head == 0)) return;    // uniform over the workgroup
-    const int pix = blockIdx.x * blockDim.x + threadIdx.x;
-    const bool active = pix < S.L;
-    int bin = 0;
-    if (active) {
-        float x, y;
-        load_xy(S.mo, S.dtype, (size_t)pix * S.h + hd, x, y);
-        bin = target_bin(S, pix, x, y);
-    }
-    count_block(S, S.count + (size_t)hd * S.nbins, S.rank + (size_t)hd * S.L + (active ? pix : 0), active, bin);
+#pragma unroll
+    for (int u = 0; u < kCountPerThread; ++u)
+        if (pix[u] < S.L) rank[pix[u]] = local[u] >= 0 ? base[bin[u] & (kCountTable - 1)] + local[u] : atomicAdd(&count[bin[u]], 1);
 }
 
 // Two-level exclusive scan of the bin counts: bins are (target row, column group), so one
