@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 # (see profiles/): filled in from the committed counter summary, None when not measured.
 # keyed by (workload, first part of the kernel name that ran)
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg3_cross", "fwd_tile_f16"): 1848822784,    # LDS-tile kernel: 2.0 x 593964 KiB fetched + 617563 KiB written
+    ("cfg3_cross", "fwd_tile_f16"): 1803636736,    # LDS-tile kernel: 2.0 x 572323 KiB fetched + 616718 KiB written
     ("cfg3_cross", "fwd_tiled_f16"): 1470390272,   # direct-gather kernel: 2.0 x 424204 KiB fetched + 587520 KiB written
     ("cfg3_cross", "fwd_tile_f32"): 3778794496,    # fp32 LDS-tile kernel: 2.0 x 1233603 KiB fetched + 1223023 KiB written
 }
