@@ -68,6 +68,9 @@ def _cold_ms(fn, reps=10):
     every call, so that no input is left in L2 or the memory-side cache by the previous call."""
     import torch
     junk = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    for _ in range(2):          # (the first call of a process loads the kernels' code: not what is measured here)
+        fn()
+    torch.cuda.synchronize()
     per = []
     for i in range(reps):
         junk.fill_(i & 0xff)

@@ -217,7 +217,7 @@ SortLayout sort_layout(int B, int H, int W, int h, int bin_w, int bin_h = 1, int
 struct TileLayout { SortLayout sl; size_t defer_off, chunk_off, item_off, total; int chunk_cap; };
 // `by_row`: the buckets are ordered by the window's row inside the tile (one sub-bucket per row), which the fp16
 // forward with 32 channels per head wants: its aggregation walks the rows the 16 queries of a wavefront reach.
-bool tile_rows_wanted(int C, int h, int dtype) { return dtype == MATCHATTN_F16 && C / h == 32; }
+bool tile_rows_wanted(int C, int h, int dtype) { return (dtype == MATCHATTN_F16 || dtype == MATCHATTN_BF16) && C / h == 32; }
 TileLayout tile_layout(int B, int H, int W, int h, bool by_row) {
     TileLayout t;
     const int sub = by_row ? ma::kTileDims[1] : 1;
@@ -291,20 +291,26 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
     const int CH = C / h, mode = O.forward_lds;
     if (mode == 0 || rx != ry || rx > 2 || O.forward_variant == 0) return false;
     // head sizes with an instance (a head group is the heads that fill a 128-byte line per pixel; 64 fp32
-    // channels would need 256-byte pixels: two workgroups' tiles no longer fit a CU's LDS)
+    // channels are 256-byte pixels: one workgroup of 512 threads per CU instead of two of 256)
     const int head_bytes = CH * (int)elem_size(dtype);
-    if (!(CH == 16 || CH == 32 || (CH == 64 && dtype != MATCHATTN_F32))) return false;
+    if (!(CH == 16 || CH == 32 || CH == 64)) return false;
     if (h % (head_bytes >= 128 ? 1 : 128 / head_bytes) != 0) return false;
     if (mode == 1) return true;
     // auto: sizes that fill the chip.  Measured against the direct gather (stereo, per-head and 2-D random fields):
     // with the 6x6 window the tiles win from about 2^20 head-queries in fp16 (5-45 % at 0.5 M pixels x 8 heads,
     // whatever the field), from 2^18 in fp32 (whose direct kernel moves twice the bytes through L2: 1.1x to 4x) and
-    // from 2^21 in bf16 (at 2^20 the stereo field still loses 10 %); with the 4x4 window from about 2^21 in fp16
-    // and fp32 (1.1x to 2x; at 2^20 the stereo field still loses 7 %), and in bf16 only on incoherent fields, so
-    // not by default.  Below that bucketing the queries costs more than it saves.
+    // from 2^20 in bf16 with 32 channels per head (the kernel that uses the matrix unit: 1.2x to 2.3x there, even at
+    // 2^19) and from 2^21 with the other head sizes (at 2^20 the stereo field still loses 10 %); with the 4x4 window
+    // from about 2^21 in fp16, fp32 and bf16 with 32 channels per head (1.1x to 2x on per-head and 2-D fields; the
+    // stereo field loses 7 % there and at 2^20 up to 16 %), and with the other bf16 head sizes only on incoherent
+    // fields, so not by default.  Below that bucketing the queries costs more than it saves.
+    // Heads of 64 fp32 channels (one workgroup of 512 threads per CU): 1.3x to 5.8x from 2^17 head-queries with the
+    // 6x6 window, 1.1x to 4.7x from 2^18 with the 4x4 window (at 2^17 the stereo field loses 18 %).
     const long long nhq = (long long)B * H * W * h;
-    if (rx == 2) return nhq >= (dtype == MATCHATTN_F32 ? (1ll << 18) : dtype == MATCHATTN_F16 ? (1ll << 20) : (1ll << 21));
-    return dtype != MATCHATTN_BF16 && nhq >= (1ll << 21);
+    if (dtype == MATCHATTN_F32 && CH == 64) return nhq >= (rx == 2 ? (1ll << 17) : (1ll << 18));
+    const bool bf_mat = dtype == MATCHATTN_BF16 && CH == 32;
+    if (rx == 2) return nhq >= (dtype == MATCHATTN_F32 ? (1ll << 18) : (dtype == MATCHATTN_F16 || bf_mat) ? (1ll << 20) : (1ll << 21));
+    return (dtype != MATCHATTN_BF16 || bf_mat) && nhq >= (1ll << 21);
 }
 }  // namespace
 
@@ -620,11 +626,13 @@ bool bwd_tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx
     const int CH = C / h, M = (2 * rx + 2) * (2 * rx + 2), mode = O.backward_mode;
     if (mode == 2 || mode == 0) return false;
     const int head_bytes = CH * (int)elem_size(dtype);
-    if (!(rx <= 2 && (CH == 16 || CH == 32 || (CH == 64 && dtype != MATCHATTN_F32)) &&
+    if (!(rx <= 2 && (CH == 16 || CH == 32 || CH == 64) &&
           h % (head_bytes >= 128 ? 1 : 128 / head_bytes) == 0 &&
           (unsigned long long)B * H * W * h * M * pair_bytes(dtype) < 0xFFFFF000ull))
         return false;
-    return mode == 1 || (long long)B * H * W * h >= (1ll << 18);   // auto: maps large enough to pay for the bucketing
+    // auto: maps large enough to pay for the bucketing (heads of 64 fp32 channels, twice the bytes per head-query: 1.1x to
+    // 1.4x at 2^17 already)
+    return mode == 1 || (long long)B * H * W * h >= ((dtype == MATCHATTN_F32 && CH == 64) ? (1ll << 17) : (1ll << 18));
 }
 BwdLayout bwd_gather_layout(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
     BwdLayout l;

@@ -11,9 +11,9 @@
 
 namespace ma {
 
-template <typename T, int CH, int R, int TW, int TH>
-__global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArgs A, TileSort S) {
-    typedef TileCfgT<T, CH, R, TW, TH, 1> Cfg;
+template <typename T, int CH, int R, int TW, int TH, int NT = kTileNT>
+__global__ __launch_bounds__(NT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArgs A, TileSort S) {
+    typedef TileCfgT<T, CH, R, TW, TH, 1, NT> Cfg;
     typedef Traits<T> Tr;
     constexpr int ES = Cfg::ES, EPV = Cfg::EPV, WN = Cfg::WN, M = Cfg::M, BW = Cfg::BW, BH = Cfg::BH;
     constexpr int GB = Cfg::GB, HPG = Cfg::HPG, CPP = Cfg::CPP, PSTR = Cfg::PSTR, LPH = Cfg::LPH, QPP = Cfg::QPP;
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void bwd_tile_kernel(BwdArg
         uint32_t src[Cfg::CPT], dst[Cfg::CPT];
 #pragma unroll
         for (int c = 0; c < Cfg::CPT; ++c) {
-            const int f = (int)threadIdx.x + c * kTileNT;
+            const int f = (int)threadIdx.x + c * NT;
             const int p = f / CPP, ch = f - p * CPP;
             const int py = p / BW, px = p - py * BW;
             const int gy = clampi(box_y + py, 0, A.H - 1), gx = clampi(box_x + px, 0, A.W - 1);

@@ -21,11 +21,12 @@ typedef bf16_t T;
 
 template <int CH, int R>
 static int launch_bwd_tile(const BwdArgs &A, const TileSort &S, hipStream_t s) {
-    typedef TileCfgT<T, CH, R, kTileW, kTileH, 1> Cfg;
+    constexpr int NT = CH * (int)sizeof(T) > 128 ? 2 * kTileNT : kTileNT;   // 256-byte heads: one workgroup of 512 per CU
+    typedef TileCfgT<T, CH, R, kTileW, kTileH, 1, NT> Cfg;
     if (A.h % Cfg::HPG != 0) return -1;
     launch_tile_chunks(S, A.h, Cfg::QPP, s);
-    const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);   // persistent: two workgroups fit a CU's LDS
-    hipLaunchKernelGGL((bwd_tile_kernel<T, CH, R, kTileW, kTileH>), dim3(grid), dim3(kTileNT), 0, s, A, S);
+    const unsigned grid = tile_grid((unsigned)Cfg::WG_PER_CU * (unsigned)kTileGridMult);   // persistent: what fits a CU's LDS
+    hipLaunchKernelGGL((bwd_tile_kernel<T, CH, R, kTileW, kTileH, NT>), dim3(grid), dim3(NT), 0, s, A, S);
     return (int)hipGetLastError();
 }
 
@@ -35,9 +36,7 @@ static int launch_bwd_tile(const BwdArgs &A, const TileSort &S, hipStream_t s) {
 int MA_CAT(launch_bwd_tile_, MA_SUFFIX)(const BwdArgs &A, const TileSort &S, int CH, int R, hipStream_t s) {
     MA_BT_CASE(16, 1) MA_BT_CASE(16, 2)
     MA_BT_CASE(32, 1) MA_BT_CASE(32, 2)
-#if MA_DTYPE != 0       // (64 fp32 channels: 256-byte pixels, the tiles of two workgroups do not fit a CU's LDS)
-    MA_BT_CASE(64, 1) MA_BT_CASE(64, 2)
-#endif
+    MA_BT_CASE(64, 1) MA_BT_CASE(64, 2)          // (64 fp32 channels: 256-byte pixels, one workgroup of 512 threads per CU)
     (void)A; (void)S; (void)s;
     return -1;
 }

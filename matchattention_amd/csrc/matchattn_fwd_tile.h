@@ -251,9 +251,15 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
     }
 }
 
-template <int CH, int R, int TW, int TH, int VPL>
+// T = half_t, or bf16_t (only in the form that runs both the L1 sums and the aggregation on the matrix unit: 32
+// channels per head).  bf16 has no packed arithmetic on this GPU: the differences are taken in fp32 from unpacked
+// halves (q is unpacked once per pass) and rounded to bf16 -- where the definition rounds them -- by the packed
+// conversion that feeds the matrix instruction; logits and weights are kept as packed bf16 pairs and unpacked by
+// shifts where the softmax needs them.
+template <int CH, int R, int TW, int TH, int VPL, typename T = half_t>
 __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(FwdArgs A, TileSort S) {
-    typedef half_t T;
+    constexpr bool kBf = std::is_same<T, bf16_t>::value;
+    static_assert(kBf || std::is_same<T, half_t>::value, "16-bit storage types");
     typedef TileCfg<CH, R, TW, TH, VPL> Cfg;
     typedef StageCfg<R, VPL> St;
     constexpr int WN = Cfg::WN, M = Cfg::M, HW = WN / 2, BW = Cfg::BW, BH = Cfg::BH;
@@ -304,9 +310,29 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     // over the 8 halves of lanes l and l ^ 16.  A lane receives rows 4 b .. 4 b + 3 of its column in its four result
     // registers; row_ones0 has its ones in the rows i % 4 == 0 only, row_ones1 in the rows i % 4 == 1, so that an
     // accumulator chained through one instruction with each keeps the two sums apart in registers 0 and 1.
-    typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+    typedef typename std::conditional<kBf, __bf16, _Float16>::type elem_t;
+    typedef elem_t half8_t __attribute__((ext_vector_type(8)));
     typedef float f32x4_t __attribute__((ext_vector_type(4)));
-    const uint32_t one_bits = (((lane_w & 15) >= 8) == (lane_w >= 32)) ? 0x3c003c00u : 0u;
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    static_assert(!kBf || (kMatrixSum && MA_TILE_MFMA_AGG && HPG == 2 && CH == 32 && BW <= 24), "bf16: the matrix-unit form only");
+    auto mfma16 = [](half8_t a, half8_t b, f32x4_t c) __attribute__((always_inline)) {
+        if constexpr (kBf) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+        else return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    };
+    // a pair of logits or weights in one register: packed halves, or packed bf16 as plain bits
+    typedef typename std::conditional<kBf, uint32_t, half2_t>::type pair_t;
+    auto pair_bits = [](pair_t p) __attribute__((always_inline)) { return __builtin_bit_cast(uint32_t, p); };
+    auto pair_of = [](uint32_t u) __attribute__((always_inline)) { return __builtin_bit_cast(pair_t, u); };
+    auto pair_lo = [](pair_t p) __attribute__((always_inline)) {
+        if constexpr (kBf) return as_f32(p << 16); else return (float)p.x;
+    };
+    auto pair_hi = [](pair_t p) __attribute__((always_inline)) {
+        if constexpr (kBf) return as_f32(p & 0xffff0000u); else return (float)p.y;
+    };
+    [[maybe_unused]] auto pack_bf16 = [](float lo, float hi) __attribute__((always_inline)) {   // both rounded to nearest even
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{lo, hi}, bf16x2_t));
+    };
+    const uint32_t one_bits = (((lane_w & 15) >= 8) == (lane_w >= 32)) ? (kBf ? 0x3f803f80u : 0x3c003c00u) : 0u;
     const uint32_t ob0 = (lane_w & 3) == 0 ? one_bits : 0u, ob1 = (lane_w & 3) == 1 ? one_bits : 0u;
     [[maybe_unused]] const half8_t row_ones0 = __builtin_bit_cast(half8_t, u32x4{ob0, ob0, ob0, ob0});
     [[maybe_unused]] const half8_t row_ones1 = __builtin_bit_cast(half8_t, u32x4{ob1, ob1, ob1, ob1});
@@ -447,8 +473,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
         for (int u = 0; u < VPL; ++u) gatev[u] = buf_load16(rgate, (uint32_t)pix * row_bytes + chan_bytes + vec_off[u]);
 
         const int hq = pix * A.h + head;
-        const half2_t xy = as_h2(xyu);
-        const float x = (float)xy.x, y = (float)xy.y;
+        const float x = pair_lo(pair_of(xyu)), y = pair_hi(pair_of(xyu));
         float x0, y0, w[4];
         corner_weights<T>(x, y, x0, y0, w);
         // centres far outside the image: every tap is a border pixel whatever the distance
@@ -481,10 +506,17 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
         typedef std::integral_constant<int, 1> VT;
 
         // ---- logits ----------------------------------------------------------------------------
-        half2_t lgp[WN][HW];
-        const half_t ninf = (half_t)(-__builtin_inff());
+        pair_t lgp[WN][HW];
+        const pair_t ninf2 = pair_of(kBf ? 0xff80ff80u : 0xfc00fc00u);       // (-inf, -inf)
 #pragma unroll
-        for (int i = 0; i < HW; ++i) lgp[WN - 1][i] = half2_t{ninf, ninf};   // stays if the row is left out
+        for (int i = 0; i < HW; ++i) lgp[WN - 1][i] = ninf2;                 // stays if the row is left out
+        [[maybe_unused]] float qf[VPL][8];                                   // bf16: q unpacked, once per pass
+        if constexpr (kBf) {
+#pragma unroll
+            for (int u = 0; u < VPL; ++u)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qf[u][e] = vec_elem<T>(qv[u], e);
+        }
         fetch(KT{}, std::integral_constant<int, 0>{});
         float held = 0.f;                               // raw sum of the even tap of a pair until its odd tap is done
         // Running sum of the raw tap sums, for one purpose: a matrix instruction multiplies the |q - k| of all four
@@ -514,9 +546,15 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                     for (int u = 0; u < VPL; ++u) {
                         u32x4 ad;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            ad[e] = h2_as_u32(as_h2(qv[u][e]) - as_h2(buf[s & 1][t][u][e])) & 0x7fff7fffu;
-                        acc4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(u == 0 ? row_ones0 : row_ones1, __builtin_bit_cast(half8_t, ad), acc4, 0, 0, 0);
+                        for (int e = 0; e < 4; ++e) {
+                            if constexpr (kBf) {
+                                const uint32_t kw = buf[s & 1][t][u][e];
+                                ad[e] = pack_bf16(qf[u][2 * e] - as_f32(kw << 16), qf[u][2 * e + 1] - as_f32(kw & 0xffff0000u)) & 0x7fff7fffu;
+                            } else {
+                                ad[e] = h2_as_u32(as_h2(qv[u][e]) - as_h2(buf[s & 1][t][u][e])) & 0x7fff7fffu;
+                            }
+                        }
+                        acc4 = mfma16(u == 0 ? row_ones0 : row_ones1, __builtin_bit_cast(half8_t, ad), acc4);
                     }
                     static_assert(!kMatrixSum || VPL == 2, "one result row per vector of a lane");
                     sum = acc4[0] + acc4[1];
@@ -533,8 +571,12 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 if (!(i & 1)) {
                     held = sum;
                     asm volatile("" : "+v"(held));
+                } else if constexpr (kBf) {
+                    const uint32_t l16 = pack_bf16(held, sum);
+                    uint32_t pinned = pack_bf16(as_f32(l16 << 16) * nscale, as_f32(l16 & 0xffff0000u) * nscale);
+                    asm volatile("" : "+v"(pinned));
+                    lgp[j][i >> 1] = pair_of(pinned);
                 } else {
-                    typedef float float2_t __attribute__((ext_vector_type(2)));
                     const half2_t l16 = __builtin_convertvector(float2_t{held, sum}, half2_t);
                     // (float)half * scale in one instruction per half: written as a fused multiply-add with a zero addend
                     // the compiler selects v_fma_mix_f32, which reads the half in place (for a plain product it converts
@@ -557,29 +599,52 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
         // result independent of that order.
         if (A.row_skip && y == y0) {
 #pragma unroll
-            for (int i = 0; i < HW; ++i) lgp[WN - 1][i] = half2_t{ninf, ninf};
+            for (int i = 0; i < HW; ++i) lgp[WN - 1][i] = ninf2;
         }
 
         // ---- window softmax (one exponential per tap around the window maximum) -------------------
         // window maximum and the maximum of the block every sub-window contains, on the packed logits
-        half2_t mall = lgp[0][0], min2[HW];
-#pragma unroll
-        for (int i = 0; i < HW; ++i) min2[i] = lgp[1][i];
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
+        float gmax, imax;
+        if constexpr (kBf) {
+            // no packed maximum for bf16: per column pair, the maxima over all rows and over the rows 1 .. 2R, unpacked
+            float call_lo[HW], call_hi[HW], cin_lo[HW], cin_hi[HW];
 #pragma unroll
             for (int i = 0; i < HW; ++i) {
-                if (j || i) mall = __builtin_elementwise_max(mall, lgp[j][i]);
-                if (j >= 2 && j <= 2 * R) min2[i] = __builtin_elementwise_max(min2[i], lgp[j][i]);
-            }
-        const float gmax = fmaxf((float)mall.x, (float)mall.y);
-        float imax = fmaxf((float)min2[0].y, (float)min2[HW - 1].x);     // columns 1 and 2R
+                cin_lo[i] = pair_lo(lgp[1][i]); cin_hi[i] = pair_hi(lgp[1][i]);
 #pragma unroll
-        for (int i = 1; i < HW - 1; ++i) imax = fmaxf(imax, fmaxf((float)min2[i].x, (float)min2[i].y));
+                for (int j = 2; j <= 2 * R; ++j) {
+                    cin_lo[i] = fmaxf(cin_lo[i], pair_lo(lgp[j][i]));
+                    cin_hi[i] = fmaxf(cin_hi[i], pair_hi(lgp[j][i]));
+                }
+                call_lo[i] = fmaxf(cin_lo[i], fmaxf(pair_lo(lgp[0][i]), pair_lo(lgp[WN - 1][i])));
+                call_hi[i] = fmaxf(cin_hi[i], fmaxf(pair_hi(lgp[0][i]), pair_hi(lgp[WN - 1][i])));
+            }
+            gmax = fmaxf(call_lo[0], call_hi[0]);
+#pragma unroll
+            for (int i = 1; i < HW; ++i) gmax = fmaxf(gmax, fmaxf(call_lo[i], call_hi[i]));
+            imax = fmaxf(cin_hi[0], cin_lo[HW - 1]);                     // columns 1 and 2R
+#pragma unroll
+            for (int i = 1; i < HW - 1; ++i) imax = fmaxf(imax, fmaxf(cin_lo[i], cin_hi[i]));
+        } else {
+            half2_t mall = lgp[0][0], min2[HW];
+#pragma unroll
+            for (int i = 0; i < HW; ++i) min2[i] = lgp[1][i];
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int i = 0; i < HW; ++i) {
+                    if (j || i) mall = __builtin_elementwise_max(mall, lgp[j][i]);
+                    if (j >= 2 && j <= 2 * R) min2[i] = __builtin_elementwise_max(min2[i], lgp[j][i]);
+                }
+            gmax = fmaxf((float)mall.x, (float)mall.y);
+            imax = fmaxf((float)min2[0].y, (float)min2[HW - 1].x);     // columns 1 and 2R
+#pragma unroll
+            for (int i = 1; i < HW - 1; ++i) imax = fmaxf(imax, fmaxf((float)min2[i].x, (float)min2[i].y));
+        }
         int far = !(gmax - imax < kSharedExpLimit);               // needs the exact per-sub-window softmax
         if constexpr (kMatrixSum) far |= !(finite_check < __builtin_inff());   // (false for NaN too)
         asm volatile("" : "+v"(far));                             // decided here, so that the logits die with the softmax
-        half2_t ap[WN][HW];
+        pair_t ap[WN][HW];
         if constexpr (kMatrixSum) {
             // Both lanes of a head-query hold all its logits.  Each takes half of the window's rows (lane `sub` rows
             // sub * HR .. sub * HR + HR - 1) through the exponentials, the row sums and the final products, and the two
@@ -598,9 +663,9 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
             for (int jj = 0; jj < HR; ++jj)
 #pragma unroll
                 for (int i = 0; i < HW; ++i) {
-                    const half2_t l2 = hi_rows ? lgp[jj + HR][i] : lgp[jj][i];
-                    e[jj][2 * i] = __builtin_amdgcn_exp2f((float)l2.x * kLog2e - gl);
-                    e[jj][2 * i + 1] = __builtin_amdgcn_exp2f((float)l2.y * kLog2e - gl);
+                    const pair_t l2 = hi_rows ? lgp[jj + HR][i] : lgp[jj][i];
+                    e[jj][2 * i] = __builtin_amdgcn_exp2f(pair_lo(l2) * kLog2e - gl);
+                    e[jj][2 * i + 1] = __builtin_amdgcn_exp2f(pair_hi(l2) * kLog2e - gl);
                 }
             // row sums over columns 0 .. WN-2 (west sub-windows) and 1 .. WN-1 (east), as subwindow_sum forms them
             float rl[HR], rr[HR];
@@ -646,7 +711,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
             for (int bb = 0; bb < 4; ++bb) c[bb] = w[bb] * __builtin_amdgcn_rcpf(ssum[bb]);
             coef9<R>(c, c9);
-            half2_t mine[HR][HW], theirs[HR][HW];
+            pair_t mine[HR][HW], theirs[HR][HW];
 #pragma unroll
             for (int jj = 0; jj < HR; ++jj) {
                 // class of my row jj among the window's rows: first, last, or in between
@@ -659,17 +724,21 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                     // product of two floats rounded once to fp16, one instruction per weight (v_fma_mixlo_f16 /
                     // v_fma_mixhi_f16, selected for a fused multiply-add with a zero addend; the plain product became a
                     // multiplication and a packed conversion: two roundings, three instructions per pair)
-                    half2_t t2;
-                    t2.x = (half_t)__builtin_fmaf(e[jj][2 * i], cr[cls<R>(2 * i)], 0.0f);
-                    t2.y = (half_t)__builtin_fmaf(e[jj][2 * i + 1], cr[cls<R>(2 * i + 1)], 0.0f);
-                    mine[jj][i] = t2;
+                    if constexpr (kBf) {
+                        mine[jj][i] = pack_bf16(e[jj][2 * i] * cr[cls<R>(2 * i)], e[jj][2 * i + 1] * cr[cls<R>(2 * i + 1)]);
+                    } else {
+                        half2_t t2;
+                        t2.x = (half_t)__builtin_fmaf(e[jj][2 * i], cr[cls<R>(2 * i)], 0.0f);
+                        t2.y = (half_t)__builtin_fmaf(e[jj][2 * i + 1], cr[cls<R>(2 * i + 1)], 0.0f);
+                        mine[jj][i] = t2;
+                    }
                 }
             }
 #pragma unroll
             for (int jj = 0; jj < HR; ++jj)
 #pragma unroll
                 for (int i = 0; i < HW; ++i)
-                    theirs[jj][i] = as_h2((uint32_t)__builtin_amdgcn_ds_swizzle((int)h2_as_u32(mine[jj][i]), kSwapHalves));
+                    theirs[jj][i] = pair_of((uint32_t)__builtin_amdgcn_ds_swizzle((int)pair_bits(mine[jj][i]), kSwapHalves));
 #pragma unroll
             for (int jj = 0; jj < HR; ++jj)
 #pragma unroll
@@ -709,7 +778,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 constexpr int NDW = M / 2, NP = NDW / 4, REM = NDW - NP * 4;
                 uint32_t dw[NDW];
 #pragma unroll
-                for (int m = 0; m < NDW; ++m) dw[m] = h2_as_u32(ap[m / HW][m % HW]);
+                for (int m = 0; m < NDW; ++m) dw[m] = pair_bits(ap[m / HW][m % HW]);
                 const uint32_t a_row = mine ? (uint32_t)pix * A.attn_row_bytes + (uint32_t)head * (uint32_t)(M * 2) : kDeadOffset;
 #pragma unroll
                 for (int t = 0; t * LPH < NP; ++t) {
@@ -765,7 +834,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
             for (int j = 0; j < WN; ++j)
 #pragma unroll
-                for (int i = 0; i < HW; ++i) wv[j][i] = sub ? h2_as_u32(ap[j][i]) >> 16 : h2_as_u32(ap[j][i]);
+                for (int i = 0; i < HW; ++i) wv[j][i] = sub ? pair_bits(ap[j][i]) >> 16 : pair_bits(ap[j][i]);
             const uint32_t wm_write = (uint32_t)((hslot * 16 + qq) * WM_ROW_BYTES + (cxv + sub) * 2);
             // (pixels 24 .. 31 of a step lie beyond the rectangle's row: those lanes read zeros, behind the V rectangle)
             uint32_t wm_read[HPG];
@@ -832,7 +901,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 for (int hg = 0; hg < HPG; ++hg)
 #pragma unroll
                     for (int cb = 0; cb < 2; ++cb)
-                        dacc[hg][cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(o.a[hg][cb], o.b[hg], dacc[hg][cb], 0, 0, 0);
+                        dacc[hg][cb] = mfma16(o.a[hg][cb], o.b[hg], dacc[hg][cb]);
             };
             load_row(std::integral_constant<int, 0>{});
             static_for<0, NT>([&](auto t_tag) __attribute__((always_inline)) {
@@ -856,7 +925,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 ov[hg] = vec_pack<T>(o8);
                 uint32_t any = 0u;                     // bit 15 / 31 set where a half has all exponent bits set
 #pragma unroll
-                for (int e = 0; e < 4; ++e) any |= (ov[hg][e] & 0x7fff7fffu) + 0x04000400u;
+                for (int e = 0; e < 4; ++e) any |= (ov[hg][e] & 0x7fff7fffu) + (kBf ? 0x00800080u : 0x04000400u);
                 const unsigned long long bad_m = __builtin_amdgcn_ballot_w64((any & 0x80008000u) != 0u);
                 ok_o[hg] = mine_o[hg] != 0 && (bad_m & col) == 0;
             }

@@ -11,8 +11,11 @@
 
 namespace ma {
 
-template <typename T, int CH, int R, int TW_, int TH_, int VPL_>
+// NT: threads per workgroup.  256 with two workgroups per CU (a head group of 128 bytes per pixel); heads of 256 bytes
+// (64 fp32 channels) take 512 threads and a CU's whole LDS: still eight wavefronts per CU, in one workgroup.
+template <typename T, int CH, int R, int TW_, int TH_, int VPL_, int NT_ = kTileNT>
 struct TileCfgT {
+    static constexpr int NT = NT_;
     static constexpr int ES = (int)sizeof(T), EPV = 16 / ES;
     static constexpr int VPL = VPL_, TW = TW_, TH = TH_;
     static constexpr int WN = 2 * R + 2, M = WN * WN;
@@ -24,11 +27,12 @@ struct TileCfgT {
     static constexpr int TILE_BYTES = BW * BH * PSTR;
     static constexpr int LPH = HB / 16 / VPL;                        // lanes per head-query (VPL x 16 bytes each)
     static_assert(HB % (16 * VPL) == 0, "head size");
-    static constexpr int QPP = kTileNT / LPH / HPG;                  // queries per head and pass
+    static constexpr int QPP = NT / LPH / HPG;                       // queries per head and pass
     static constexpr int NCHUNK = BW * BH * CPP;
-    static constexpr int CPT = (NCHUNK + kTileNT - 1) / kTileNT;
+    static constexpr int CPT = (NCHUNK + NT - 1) / NT;
     static_assert(LPH == 1 || LPH == 2 || LPH == 4 || LPH == 8 || LPH == 16, "head size");
-    static_assert(2 * TILE_BYTES <= 80 * 1024, "K and V tiles of two workgroups must fit a CU's LDS");
+    static constexpr int WG_PER_CU = 2 * kTileNT / NT;               // eight wavefronts per CU
+    static_assert(WG_PER_CU >= 1 && 2 * TILE_BYTES * WG_PER_CU + 1024 <= 160 * 1024, "K and V tiles of a CU's workgroups must fit its LDS");
     static_assert(kTileCap % QPP == 0, "a chunk is a whole number of passes");
 };
 
@@ -58,9 +62,9 @@ __device__ __forceinline__ void position_xy(const RawPosition<T> &p, float &x, f
     }
 }
 
-template <typename T, int CH, int R, int TW, int TH, int VPL>
-__global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArgs A, TileSort S) {
-    typedef TileCfgT<T, CH, R, TW, TH, VPL> Cfg;
+template <typename T, int CH, int R, int TW, int TH, int VPL, int NT = kTileNT>
+__global__ __launch_bounds__(NT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArgs A, TileSort S) {
+    typedef TileCfgT<T, CH, R, TW, TH, VPL, NT> Cfg;
     typedef StageCfg<R, VPL> St;
     typedef Traits<T> Tr;
     constexpr int ES = Cfg::ES, EPV = Cfg::EPV, WN = Cfg::WN, M = Cfg::M, BW = Cfg::BW, BH = Cfg::BH;
@@ -137,7 +141,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_tile_kernel(FwdArg
     uint32_t src[Cfg::CPT], dst[Cfg::CPT];
 #pragma unroll
     for (int c = 0; c < Cfg::CPT; ++c) {
-        const int f = (int)threadIdx.x + c * kTileNT;
+        const int f = (int)threadIdx.x + c * NT;
         const int p = f / CPP, ch = f - p * CPP;
         const int py = p / BW, px = p - py * BW;
         const int gy = clampi(box_y + py, 0, A.H - 1), gx = clampi(box_x + px, 0, A.W - 1);

@@ -24,12 +24,18 @@ typedef bf16_t T;
 template <int CH, int R>
 static int launch_tile(const FwdArgs &A, const TileSort &S, hipStream_t s) {
     constexpr int VPL = CH * (int)sizeof(T) >= 32 ? 2 : 1;            // vectors per lane
-    typedef TileCfgT<T, CH, R, kTileW, kTileH, VPL> Cfg;
+    constexpr int NT = CH * (int)sizeof(T) > 128 ? 2 * kTileNT : kTileNT;   // 256-byte heads: one workgroup of 512 per CU
+    typedef TileCfgT<T, CH, R, kTileW, kTileH, VPL, NT> Cfg;
     if (A.h % Cfg::HPG != 0) return -1;
     launch_tile_chunks(S, A.h, Cfg::QPP, s);
-    const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);   // persistent: two workgroups fit a CU's LDS
+    const unsigned grid = tile_grid((unsigned)Cfg::WG_PER_CU * (unsigned)kTileGridMult);   // persistent: what fits a CU's LDS
     timer_mark(false, s);
-    hipLaunchKernelGGL((fwd_tile_kernel<T, CH, R, kTileW, kTileH, VPL>), dim3(grid), dim3(kTileNT), 0, s, A, S);
+#if MA_DTYPE == 2
+    // 32 bf16 channels per head: the 16-bit kernel with its sums and its aggregation on the matrix unit
+    if constexpr (CH == 32) hipLaunchKernelGGL((fwd_h16_tile_kernel<CH, R, kTileW, kTileH, 2, bf16_t>), dim3(grid), dim3(kTileNT), 0, s, A, S);
+    else
+#endif
+    hipLaunchKernelGGL((fwd_tile_kernel<T, CH, R, kTileW, kTileH, VPL, NT>), dim3(grid), dim3(NT), 0, s, A, S);
     timer_mark(true, s);
     return (int)hipGetLastError();
 }
@@ -43,9 +49,7 @@ static int launch_tile(const FwdArgs &A, const TileSort &S, hipStream_t s) {
 int MA_CAT(launch_fwd_tile_, MA_SUFFIX)(const FwdArgs &A, const TileSort &S, int CH, int R, hipStream_t s, const char **name) {
     MA_TILE_CASE(16, 1) MA_TILE_CASE(16, 2)
     MA_TILE_CASE(32, 1) MA_TILE_CASE(32, 2)
-#if MA_DTYPE != 0       // (64 fp32 channels: K and V tiles of 256-byte pixels do not fit two workgroups per CU)
-    MA_TILE_CASE(64, 1) MA_TILE_CASE(64, 2)
-#endif
+    MA_TILE_CASE(64, 1) MA_TILE_CASE(64, 2)      // (64 fp32 channels: 256-byte pixels, one workgroup of 512 threads per CU)
     (void)A; (void)S; (void)s; (void)name;
     return -1;
 }
