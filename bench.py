@@ -412,6 +412,9 @@ def main():
                 rec["bwd_ms"] = round(ms, 4)
                 rec["bwd_GBps"] = round(w2.backward_bytes(i2["d_attn"] is not None) / (ms * 1e-3) / 1e9, 1)
                 rec["bwd_kernel"] = _cabi.last_backward_kernel()
+                tr = MEASURED_BWD_TRAFFIC_BYTES.get((name, rec["bwd_kernel"]))
+                if tr:      # HBM-side bytes per kernel of the call (counters, profiles/bwd_gather_cfg4_cfg2.md)
+                    rec["bwd_traffic"] = dict(tr, algorithmic_bytes=w2.backward_bytes(i2["d_attn"] is not None))
                 del k3
             if name in ("cfg3_cross", "cfg2_cross"):
                 rec["module_step"] = _module_step_ms(w2, i2)
@@ -431,20 +434,25 @@ def main():
             torch.cuda.empty_cache()
 
     if not args.no_extra:
-        # the same headline workload with a spatially smooth offset field (blurred to sigma = 8 px)
-        i3 = make_inputs(wl, smooth=True)
-        rec = {}
-        for tag, lds in (("fwd_ms", -1), ("fwd_direct_ms", 0)):
-            _cabi.set_option("forward_lds", lds)
-            try:
-                c5, k5 = _forward_call(lib, wl, i3)
-                _, ms, _ = _events_ms(c5, max(5, args.steps // 5), 3)
-                rec[tag] = round(ms, 4)
-                del k5
-            finally:
-                _cabi.set_option("forward_lds", -1)
-        extra[args.workload + "_smooth_field"] = rec
-        del i3
+        # the same headline workload with other offset fields: the i.i.d. one blurred to sigma = 8 px at the same amplitude
+        # (correlated, but the offsets still change by several pixels per pixel), and a field as a stereo scene gives it
+        # (slanted surfaces and discontinuities: the offsets of neighbours differ by a fraction of a pixel)
+        for field_tag, kind in (("_smooth_field", True), ("_scene_field", "scene")):
+            if kind == "scene" and not wl.offsets.startswith("stereo"):
+                continue
+            i3 = make_inputs(wl, smooth=kind)
+            rec = {}
+            for tag, lds in (("fwd_ms", -1), ("fwd_direct_ms", 0)):
+                _cabi.set_option("forward_lds", lds)
+                try:
+                    c5, k5 = _forward_call(lib, wl, i3)
+                    _, ms, _ = _events_ms(c5, max(5, args.steps // 5), 3)
+                    rec[tag] = round(ms, 4)
+                    del k5
+                finally:
+                    _cabi.set_option("forward_lds", -1)
+            extra[args.workload + field_tag] = rec
+            del i3
         # the largest maps in the other storage types (fp32 is the reference script's default precision)
         import dataclasses
         for name in ("cfg3_cross", "cfg3_self"):

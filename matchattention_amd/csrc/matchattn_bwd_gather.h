@@ -138,19 +138,19 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if constexpr (std::is_same<T, half_t>::value) {
-                // packed fp16 difference (exact sign); sgn(d) stays packed in half precision -- two multiplications by
-                // 2^15 lift the smallest subnormal difference (2^-24) above 1, the clamp to [-1, 1] leaves 0, 1.0 or
-                // -1.0 -- and the multiply-adds read it, and dO, as their half-precision operands
-                const half2_t lift = {(half_t)32768.0f, (half_t)32768.0f}, one = {(half_t)1.0f, (half_t)1.0f};
+                // packed fp16 difference (exact sign); sgn(d) per element as in pass A: the half times 2^60 in one
+                // mixed-precision instruction, the median of (x, -1, 1), a plain fp32 multiply-add; dO is read by its
+                // multiply-add as a half-precision operand
 #pragma unroll
                 for (int w = 0; w < VPL; ++w)
 #pragma unroll
                     for (int p2 = 0; p2 < 4; ++p2) {
                         const half2_t d = as_h2(bt.qv[u][w][p2]) - as_h2(kv[w][p2]);
-                        const half2_t sg = __builtin_elementwise_min(__builtin_elementwise_max((d * lift) * lift, -one), one);
                         const half2_t gp = as_h2(bt.gv[u][w][p2]);
-                        dk[w][2 * p2] = __builtin_fmaf((float)sg.x, bt.dl[u], dk[w][2 * p2]);
-                        dk[w][2 * p2 + 1] = __builtin_fmaf((float)sg.y, bt.dl[u], dk[w][2 * p2 + 1]);
+                        const float s0 = __builtin_amdgcn_fmed3f(__builtin_fmaf((float)d.x, 0x1p60f, 0.0f), -1.0f, 1.0f);
+                        const float s1 = __builtin_amdgcn_fmed3f(__builtin_fmaf((float)d.y, 0x1p60f, 0.0f), -1.0f, 1.0f);
+                        dk[w][2 * p2] = __builtin_fmaf(s0, bt.dl[u], dk[w][2 * p2]);
+                        dk[w][2 * p2 + 1] = __builtin_fmaf(s1, bt.dl[u], dk[w][2 * p2 + 1]);
                         dv[w][2 * p2] += bt.am[u] * (float)gp.x;
                         dv[w][2 * p2 + 1] += bt.am[u] * (float)gp.y;
                     }

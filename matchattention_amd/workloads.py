@@ -1,6 +1,8 @@
 """Synthetic operator workloads: the shapes and offset distributions the benchmark and
 the full-size tests use.  Inputs are i.i.d. per pixel as specified (no spatial coherence),
-which is the hardest case for tap reuse; `smooth=True` blurs the offset field instead."""
+which is the hardest case for tap reuse; `smooth=True` blurs the offset field instead (same amplitude, correlated over
+about 8 px: still several pixels of offset change per pixel), `smooth="scene"` makes a stereo field as a scene gives it
+(slanted surfaces with discontinuities: a fraction of a pixel of change per pixel).  """
 from dataclasses import dataclass
 from typing import Optional
 
@@ -103,7 +105,19 @@ def make_inputs(wl: Workload, device="cuda", seed: Optional[int] = None, smooth:
         rpos[..., 0] = -torch.rand(wl.B, N, hh, generator=g, device=device) * float(val)
     else:
         rpos = randn(wl.B, N, hh, 2) * float(val)
-    if smooth:  # spatially coherent field: box-blur the i.i.d. one a few times (about sigma 8 px)
+    if smooth == "scene" and kind == "stereo":
+        # a field as a stereo scene gives it: disparity a coarse random grid (cells of 256 px) upsampled bicubically to
+        # the map (mean |d disparity / dx| about 0.35 px per px) with three foreground boxes 25-40 px nearer on top
+        # (discontinuities); the same for every head and image
+        cell = 256
+        coarse = torch.rand(1, 1, H // cell + 2, wl.W // cell + 2, generator=g, device=device)
+        d = torch.nn.functional.interpolate(coarse, size=(H, wl.W), mode="bicubic", align_corners=True).clamp(0, 1)[0, 0]
+        d = d * (float(val) * 5.0 / 6.0)
+        for fy0, fy1, fx0, fx1, dd in ((0.18, 0.55, 0.21, 0.44, 1 / 6), (0.64, 0.92, 0.62, 0.83, 5 / 48), (0.09, 0.28, 0.73, 0.94, 1 / 8)):
+            d[int(fy0 * H):int(fy1 * H), int(fx0 * wl.W):int(fx1 * wl.W)] += dd * float(val)
+        rpos = torch.zeros(wl.B, N, hh, 2, device=device)
+        rpos[..., 0] = -d.reshape(1, N, 1)
+    elif smooth:  # spatially correlated field: box-blur the i.i.d. one a few times (about sigma 8 px)
         f = rpos.view(wl.B, H, wl.W, hh * 2).permute(0, 3, 1, 2)
         amp = f.std().clamp_min(1e-6)
         for _ in range(3):

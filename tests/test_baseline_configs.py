@@ -18,10 +18,10 @@ pytestmark = pytest.mark.gpu
 
 
 
-def _inputs(name):
+def _inputs(name, field=False):
     from matchattention_amd.workloads import WORKLOADS, make_inputs
     wl = WORKLOADS[name]
-    return wl, make_inputs(wl)
+    return wl, make_inputs(wl, smooth=field)
 
 
 def test_cfg1_forward_whole_map(hip_lib):
@@ -74,9 +74,16 @@ def test_cfg4_backward_whole_map(hip_lib, name):
         check_err(a, b, GRAD_TOL[torch.float16], f"{name} bwd {tensor} f16")
 
 
-@pytest.mark.parametrize("name", ["cfg3_cross", "cfg3_self", "cfg4_cross", "cfg4_self"])
-def test_large_maps_forward_whole_map(hip_lib, name):
-    wl, inp = _inputs(name)
+@pytest.mark.parametrize("name,field,dt", [
+    ("cfg3_cross", False, None), ("cfg3_self", False, None), ("cfg4_cross", False, None), ("cfg4_self", False, None),
+    # spatially coherent offsets (a stereo scene's field: what a model's cross-attention produces), and bfloat16
+    ("cfg3_cross", "scene", None), ("cfg3_cross", False, torch.bfloat16)],
+    ids=["cfg3_cross", "cfg3_self", "cfg4_cross", "cfg4_self", "cfg3_cross_scene_field", "cfg3_cross_bf16"])
+def test_large_maps_forward_whole_map(hip_lib, name, field, dt):
+    wl, inp = _inputs(name, field)
+    if dt is not None:
+        for n in ("max_offset", "q", "k", "v"):
+            inp[n] = inp[n].to(dt)
     H, W = inp["H"], inp["W"]
     out, attn = hip_forward(hip_lib, inp["max_offset"], inp["q"], inp["k"], inp["v"], H, W, wl.r, wl.scale)
     # A second run puts the head-queries into other lanes (the order inside a bucket is first come, first served) and
@@ -91,8 +98,8 @@ def test_large_maps_forward_whole_map(hip_lib, name):
     del inp
     torch.cuda.empty_cache()
     want_out, want_attn = O.forward_chunked(*cpu, H, W, [wl.r, wl.r], wl.scale, rows_per_chunk=8)
-    check_err(attn, want_attn, TOL[dt], f"{name} fwd attn f16")
-    check_err(out, want_out, TOL[dt], f"{name} fwd out f16")
+    check_err(attn, want_attn, TOL[dt], f"{name} fwd attn {dt}")
+    check_err(out, want_out, TOL[dt], f"{name} fwd out {dt}")
 
 
 def test_map_with_more_tiles_than_a_thread_keeps(hip_lib):

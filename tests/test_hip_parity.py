@@ -243,14 +243,16 @@ def test_full_size_tile_path_in_fp32_and_bf16(hip_lib, dt):
     assert float((res[-1][1].float().sum(-1) - 1).abs().max()) <= {torch.float32: 1e-5, torch.bfloat16: 4e-2}[dt]
 
 
-@pytest.mark.parametrize("name", ["cfg3_cross", "cfg4_self"])
-def test_full_size_tile_and_direct_paths_agree(hip_lib, name):
+@pytest.mark.parametrize("name,field", [("cfg3_cross", False), ("cfg4_self", False), ("cfg3_cross", "scene"), ("cfg3_cross", True)],
+                         ids=["cfg3_cross", "cfg4_self", "cfg3_cross_scene_field", "cfg3_cross_smooth_field"])
+def test_full_size_tile_and_direct_paths_agree(hip_lib, name, field):
     # at the benchmark's full sizes the oracle is too slow: the two HIP paths (LDS tiles / direct gather) must
-    # agree with each other, attention rows must sum to one and a constant V must come back unchanged
+    # agree with each other, attention rows must sum to one and a constant V must come back unchanged -- on the
+    # i.i.d. fields of the benchmark and on spatially coherent ones (a stereo scene's, and the blurred field)
     from matchattention_amd import _cabi
     from matchattention_amd.workloads import WORKLOADS, make_inputs
     wl = WORKLOADS[name]
-    inp = make_inputs(wl)
+    inp = make_inputs(wl, smooth=field)
     H, W = inp["H"], inp["W"]
     res = {}
     left = []
