@@ -32,7 +32,11 @@ __device__ __forceinline__ void tap_interval(int c, int key, int n, int R, int W
 // further (6 or 8 waves) spills.
 template <typename T, int CH, int R> struct KeyVpl { static constexpr int value = 1; };
 
-template <typename T, int CH, int R, int VPL>
+// COMPACT (maps below 2^25 pixels whose pair array stays below 4 GiB: chosen by the host): away from the border a
+// prepared candidate travels as one word, (query pixel << 6) | tap, or -1 for none -- one lane exchange instead of two
+// and nothing to unpack -- and its pair is fetched through a buffer descriptor, whose range check stands in for the
+// selects a missing candidate otherwise needs (an offset beyond the array reads zeros).
+template <typename T, int CH, int R, int VPL, bool COMPACT>
 __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
     typedef TiledCfg<T, CH, R, VPL> Cfg;
     constexpr int EPV = Cfg::EPV, LPH = Cfg::LPH, WN = Cfg::WN, M = Cfg::M;
@@ -59,6 +63,8 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
     const __amdgpu_buffer_rsrc_t rq = make_rsrc(A.q, total_bytes);
     const __amdgpu_buffer_rsrc_t rk = make_rsrc(A.k, total_bytes);
     const __amdgpu_buffer_rsrc_t rg = make_rsrc(A.d_out, total_bytes);
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t rp =
+        make_rsrc(A.dl_ws, COMPACT ? (uint32_t)A.nhq * (uint32_t)(M * PairOf<T>::kBytes) : 0u);
 
     u32x4 kv[VPL];
     float dk[VPL][EPV], dv[VPL][EPV];
@@ -134,6 +140,13 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
         const bool hit = t0 + gl < total && i_lo <= i_hi && j_lo <= j_hi;
         return hit ? (1 << 12) | (j_hi << 9) | (j_lo << 6) | (i_hi << 3) | i_lo : 0;
     };
+    // the same for a key away from the border, as one word: (query pixel << 6) | tap, or -1
+    [[maybe_unused]] auto make_word = [&](int t0, int cc, int qp) __attribute__((always_inline)) {
+        const int cx = (int)(int16_t)(cc & 0xffff), cy = cc >> 16;
+        const int i = kx - cx + R, j = ky - cy + R;
+        const bool hit = t0 + gl < total && i >= 0 && i < WN && j >= 0 && j < WN;
+        return hit ? (qp << 6) | (j * WN + i) : -1;
+    };
     auto sum = [&](const Batch &bt) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -169,16 +182,18 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
     // cannot count the loads in flight and waits for all of them before every batch)
     auto walk = [&](auto one_tap_tag) __attribute__((always_inline)) {
         constexpr bool ONE = decltype(one_tap_tag)::value;
+        constexpr bool PACKED = ONE && COMPACT;
         int t0 = 0, tf = 0;                            // start of the prepared chunk; next candidate to fetch
         int qp_m, cc_m, qp_n, cc_n;
         { const int p = locate(gl); qp_m = clampi(perm[p], 0, npix - 1); cc_m = centre[p]; }
         { const int p = locate(GW + gl); qp_n = perm[p]; cc_n = centre[p]; }
-        int info_m = make_info(0, cc_m);
+        int info_m;
+        if constexpr (PACKED) info_m = make_word(0, cc_m, qp_m); else info_m = make_info(0, cc_m);
         auto fetch = [&](Batch &bt) __attribute__((always_inline)) {
             if (tf >= t0 + GW) {                       // the chunk is used up (the same for the whole group): next one,
                 t0 += GW;                              // and the index entries of the one after it go in flight
                 qp_m = clampi(qp_n, 0, npix - 1);
-                info_m = make_info(t0, cc_n);
+                if constexpr (PACKED) info_m = make_word(t0, cc_n, qp_m); else info_m = make_info(t0, cc_n);
                 const int p = locate(t0 + GW + gl);
                 qp_n = perm[p]; cc_n = centre[p];
             }
@@ -186,6 +201,23 @@ __global__ __launch_bounds__(256) void bwd_key_kernel(BwdArgs A) {
             for (int u = 0; u < U; ++u) {
                 const int idx = tf + u - t0;
                 const int from = (gb + min(idx, GW - 1)) * 4;
+                if constexpr (PACKED) {
+                    const int word = u < step ? __builtin_amdgcn_ds_bpermute(from, info_m) : -1;
+                    const bool hit = word >= 0;
+                    const uint32_t qp = (uint32_t)word >> 6;
+                    const uint32_t poff = hit ? pairs.at(qp, (uint32_t)word & 63u) * (uint32_t)PairOf<T>::kBytes : kDeadOffset;
+                    typename PairOf<T>::Word da;
+                    if constexpr (PairOf<T>::kBytes == 4) da = (typename PairOf<T>::Word)__builtin_amdgcn_raw_buffer_load_b32(rp, (int)poff, 0, 0);
+                    else da = __builtin_amdgcn_raw_buffer_load_b64(rp, (int)poff, 0, 0);
+                    PairOf<T>::unpack(da, bt.dl[u], bt.am[u]);
+                    const uint32_t off = (carries && hit) ? qp * row_bytes + chan_bytes : kDeadOffset;
+#pragma unroll
+                    for (int w = 0; w < VPL; ++w) {
+                        bt.qv[u][w] = buf_load16(rq, off + w * 16);
+                        bt.gv[u][w] = buf_load16(rg, off + w * 16);
+                    }
+                    continue;
+                }
                 const int qp = __builtin_amdgcn_ds_bpermute(from, qp_m);
                 const int info = (u < step && tf + u < total) ? __builtin_amdgcn_ds_bpermute(from, info_m) : 0;
                 const bool hit = (info >> 12) != 0;

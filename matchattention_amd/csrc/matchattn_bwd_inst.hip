@@ -59,7 +59,10 @@ static int launch_key(const BwdArgs &A, hipStream_t s) {
     constexpr int VPL = KeyVpl<T, CH, R>::value;
     typedef TiledCfg<T, CH, R, VPL> Cfg;
     const unsigned nblocks = (unsigned)((A.nhq + Cfg::HQ_PER_BLOCK - 1) / Cfg::HQ_PER_BLOCK);
-    hipLaunchKernelGGL((bwd_key_kernel<T, CH, R, VPL>), dim3(nblocks), dim3(Cfg::BLOCK), 0, s, A);
+    // (the compact form of a candidate: the pixel index in 25 bits, the pair array within a buffer descriptor's 4 GiB)
+    const bool compact = A.nhq / A.h < (1 << 25) && (unsigned long long)A.nhq * Cfg::M * PairOf<T>::kBytes < 0xFFFFF000ull;
+    if (compact) hipLaunchKernelGGL((bwd_key_kernel<T, CH, R, VPL, true>), dim3(nblocks), dim3(Cfg::BLOCK), 0, s, A);
+    else hipLaunchKernelGGL((bwd_key_kernel<T, CH, R, VPL, false>), dim3(nblocks), dim3(Cfg::BLOCK), 0, s, A);
     return (int)hipGetLastError();
 }
 
