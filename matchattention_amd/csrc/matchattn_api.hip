@@ -296,21 +296,23 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
     if (!(CH == 16 || CH == 32 || CH == 64)) return false;
     if (h % (head_bytes >= 128 ? 1 : 128 / head_bytes) != 0) return false;
     if (mode == 1) return true;
-    // auto: sizes that fill the chip.  Measured against the direct gather (stereo, per-head and 2-D random fields):
-    // with the 6x6 window the tiles win from about 2^20 head-queries in fp16 (5-45 % at 0.5 M pixels x 8 heads,
-    // whatever the field), from 2^18 in fp32 (whose direct kernel moves twice the bytes through L2: 1.1x to 4x) and
-    // from 2^20 in bf16 with 32 channels per head (the kernel that uses the matrix unit: 1.2x to 2.3x there, even at
-    // 2^19) and from 2^21 with the other head sizes (at 2^20 the stereo field still loses 10 %); with the 4x4 window
-    // from about 2^21 in fp16, fp32 and bf16 with 32 channels per head (1.1x to 2x on per-head and 2-D fields; the
-    // stereo field loses 7 % there and at 2^20 up to 16 %), and with the other bf16 head sizes only on incoherent
-    // fields, so not by default.  Below that bucketing the queries costs more than it saves.
+    // auto: sizes that fill the chip.  Measured against the direct gather (stereo, per-head and 2-D random fields, 8 and
+    // 16 heads, one process): with the 6x6 window the tiles win from about 2^19 head-queries with 32 16-bit channels per
+    // head (the kernel that uses the matrix unit; fp16 1.3x to 2.2x at 2^19, 0.75x to 1.3x at 2^18; bf16 1.1x to 2.2x and
+    // 0.9x to 1.7x), from 2^20 with the other fp16 head sizes, from 2^18 in fp32 (whose direct kernel moves twice the
+    // bytes through L2: 1.1x to 4x) and from 2^21 with the other bf16 head sizes (at 2^20 the stereo field still loses
+    // 10 %); with the 4x4 window from 2^20 in fp16 with 32 channels per head (1.07x to 1.9x; at 2^19 the stereo field
+    // loses 13 %), from about 2^21 with the other fp16 head sizes, in fp32 and in bf16 with 32 channels per head (1.5x to
+    // 2x on per-head and 2-D fields; the bf16 stereo field loses 4 % there), and with the other bf16 head sizes only on
+    // incoherent fields, so not by default.  Below that bucketing the queries costs more than it saves.
     // Heads of 64 fp32 channels (one workgroup of 512 threads per CU): 1.3x to 5.8x from 2^17 head-queries with the
     // 6x6 window, 1.1x to 4.7x from 2^18 with the 4x4 window (at 2^17 the stereo field loses 18 %).
     const long long nhq = (long long)B * H * W * h;
     if (dtype == MATCHATTN_F32 && CH == 64) return nhq >= (rx == 2 ? (1ll << 17) : (1ll << 18));
-    const bool bf_mat = dtype == MATCHATTN_BF16 && CH == 32;
-    if (rx == 2) return nhq >= (dtype == MATCHATTN_F32 ? (1ll << 18) : (dtype == MATCHATTN_F16 || bf_mat) ? (1ll << 20) : (1ll << 21));
-    return (dtype != MATCHATTN_BF16 || bf_mat) && nhq >= (1ll << 21);
+    const bool mat16 = dtype != MATCHATTN_F32 && CH == 32;        // fwd_h16_tile_kernel with its matrix-unit phases
+    if (rx == 2) return nhq >= (dtype == MATCHATTN_F32 ? (1ll << 18) : mat16 ? (1ll << 19) : dtype == MATCHATTN_F16 ? (1ll << 20) : (1ll << 21));
+    if (mat16 && dtype == MATCHATTN_F16) return nhq >= (1ll << 20);
+    return (dtype != MATCHATTN_BF16 || mat16) && nhq >= (1ll << 21);
 }
 }  // namespace
 

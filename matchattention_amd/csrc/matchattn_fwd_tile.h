@@ -66,6 +66,10 @@ constexpr int kTileCap = MA_TILE_CAP;
 #define MA_TILE_GRID_MULT 2
 #endif
 constexpr int kTileGridMult = MA_TILE_GRID_MULT;
+// 1: the bf16 forward subtracts q - k on the matrix unit (fwd_h16_tile_kernel, K phase)
+#ifndef MA_TILE_BF16_MFMA_SUB
+#define MA_TILE_BF16_MFMA_SUB 1
+#endif
 // 1: the fp16 forward with 32 channels per head aggregates on the matrix unit (fwd_h16_tile_kernel, V phase)
 #ifndef MA_TILE_MFMA_AGG
 #define MA_TILE_MFMA_AGG 1
@@ -336,6 +340,23 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     const uint32_t ob0 = (lane_w & 3) == 0 ? one_bits : 0u, ob1 = (lane_w & 3) == 1 ? one_bits : 0u;
     [[maybe_unused]] const half8_t row_ones0 = __builtin_bit_cast(half8_t, u32x4{ob0, ob0, ob0, ob0});
     [[maybe_unused]] const half8_t row_ones1 = __builtin_bit_cast(half8_t, u32x4{ob1, ob1, ob1, ob1});
+    // bf16: the subtraction q - k itself runs on the matrix unit (v_mfma_f32_16x16x16_bf16: four elements per lane and
+    // operand).  With four K values of each of the 64 lanes as the B operand (lane j + 16 b: column j, rows 4 b .. 4 b + 3)
+    // and an A operand that holds a single -1 per row -- A[4 b + r][4 b + r] -- result row 4 b + r of column j is minus
+    // element r of lane j + 16 b's own four: every lane gets its own four K values back, widened to fp32 and negated,
+    // added to the C operand, which holds the same four elements of q (unpacked once per pass).  Two instructions per
+    // vector and tap replace the two unpacking and two subtracting vector instructions per word -- there is no packed
+    // bf16 arithmetic -- and leave the vector ALU the rounding of the differences to bf16 and the sign mask, as in
+    // fp16.  (0 x inf = NaN reaches the other lanes of a column, as with the sums: such head-queries are left to the
+    // generic kernel.)
+    typedef short short4v_t __attribute__((ext_vector_type(4)));
+    [[maybe_unused]] short4v_t sel_neg = {0, 0, 0, 0};
+    if constexpr (kBf && MA_TILE_BF16_MFMA_SUB) {
+        const bool diag = (lane_w >> 4) == ((lane_w & 15) >> 2);
+        const short m1 = (short)0xbf80;                  // -1.0 in bf16
+        sel_neg = short4v_t{(short)(diag && (lane_w & 3) == 0 ? m1 : 0), (short)(diag && (lane_w & 3) == 1 ? m1 : 0),
+                            (short)(diag && (lane_w & 3) == 2 ? m1 : 0), (short)(diag && (lane_w & 3) == 3 ? m1 : 0)};
+    }
     // Lane `sub` owns the 16-byte vectors sub, sub + LPH, ... of its head, so that the lanes of one LDS read
     // touch adjacent 16-byte pieces (vectors 2 sub, 2 sub + 1 would put them 32 bytes apart: 2-way bank
     // conflicts).  With two vectors per lane, odd lane groups take theirs in the opposite order: one LDS
@@ -545,6 +566,17 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
                     for (int u = 0; u < VPL; ++u) {
                         u32x4 ad;
+                        if constexpr (kBf && MA_TILE_BF16_MFMA_SUB) {
+                            const u32x4 kw = buf[s & 1][t][u];
+                            const f32x4_t d0 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sel_neg, __builtin_bit_cast(short4v_t, u32x2{kw[0], kw[1]}),
+                                                                                         f32x4_t{qf[u][0], qf[u][1], qf[u][2], qf[u][3]}, 0, 0, 0);
+                            const f32x4_t d1 = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(sel_neg, __builtin_bit_cast(short4v_t, u32x2{kw[2], kw[3]}),
+                                                                                         f32x4_t{qf[u][4], qf[u][5], qf[u][6], qf[u][7]}, 0, 0, 0);
+                            ad[0] = pack_bf16(d0[0], d0[1]) & 0x7fff7fffu;
+                            ad[1] = pack_bf16(d0[2], d0[3]) & 0x7fff7fffu;
+                            ad[2] = pack_bf16(d1[0], d1[1]) & 0x7fff7fffu;
+                            ad[3] = pack_bf16(d1[2], d1[3]) & 0x7fff7fffu;
+                        } else
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             if constexpr (kBf) {
