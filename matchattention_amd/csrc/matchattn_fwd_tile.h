@@ -545,8 +545,10 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
         // overflows fp16) of one head-query would turn the logits of the unrelated head-query in lanes l ^ 32 into NaN
         // as well.  The sums are >= 0, so the total is finite exactly when every one of them was; head-queries whose
         // total is not are left to the generic kernel, which keeps such values local to the query that owns them.
-        // (Not needed where the aggregation runs on the matrix unit as well: a NaN logit makes every weight of its
-        // head-query NaN, hence its output, and the aggregation's own check of the results hands it over.)
+        // (Where the aggregation runs on the matrix unit as well, only the last window row needs it: a NaN logit makes
+        // every weight of its head-query NaN, hence its output, and the aggregation's own check of the results hands it
+        // over -- except in the row a lane with integer y drops after the wavefront has computed it, which the generic
+        // kernel would multiply by its zero weight: NaN there, lost here.)
         [[maybe_unused]] float finite_check = 0.f;
         static_for<0, NSR>([&](auto s_tag) __attribute__((always_inline)) {
             constexpr int s = decltype(s_tag)::value, j = s / SPR, i0 = (s % SPR) * G;
@@ -592,7 +594,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                     }
                     static_assert(!kMatrixSum || VPL == 2, "one result row per vector of a lane");
                     sum = acc4[0] + acc4[1];
-                    if constexpr (!kMatrixAgg) finite_check += sum;
+                    if constexpr (!kMatrixAgg || j == WN - 1) finite_check += sum;
                 } else {
                     sum = l1_sum<T>(qv[0], buf[s & 1][t][0]);
 #pragma unroll
@@ -676,7 +678,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
             for (int i = 1; i < HW - 1; ++i) imax = fmaxf(imax, fmaxf((float)min2[i].x, (float)min2[i].y));
         }
         int far = !(gmax - imax < kSharedExpLimit);               // needs the exact per-sub-window softmax
-        if constexpr (kMatrixSum && !kMatrixAgg) far |= !(finite_check < __builtin_inff());   // (false for NaN too)
+        if constexpr (kMatrixSum) far |= !(finite_check < __builtin_inff());   // (false for NaN too)
         asm volatile("" : "+v"(far));                             // decided here, so that the logits die with the softmax
         pair_t ap[WN][HW];
         if constexpr (kMatrixSum) {

@@ -726,10 +726,18 @@ def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib, dt, big):
         assert rel_err(b[0, keep].float().cpu(), a[0, keep].float().cpu()) <= TOL[dt]
         same = (a[0, keep] == b[0, keep]).flatten(1).all(1).float().mean().item()
         assert same >= 0.95, same
-    # the queries that own a poisoned value get what the kernels without a matrix unit give them
-    for a, b in zip(bad, direct):
-        own = touched.cuda()
-        assert torch.equal(torch.isfinite(a[0, own]), torch.isfinite(b[0, own]))
+    # the queries that own a poisoned value get what the kernels without a matrix unit give them -- in every run: which
+    # queries share a wavefront changes from call to call, and what an owner gets must not (one of them has an integer
+    # y and its NaN in the window row such a lane drops)
+    own = touched.cuda()
+    for _ in range(6):
+        for a, b in zip(bad, direct):
+            assert torch.equal(torch.isfinite(a[0, own]), torch.isfinite(b[0, own]))
+        try:
+            _cabi.set_option("forward_lds", 1)
+            bad = hip_forward(hip_lib, *_dev(mo, qb, kb, v), H, W, r, 0.2)
+        finally:
+            _cabi.set_option("forward_lds", -1)
 
 
 def test_bf16_backward_keeps_small_gradients(hip_lib):
