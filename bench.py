@@ -46,6 +46,68 @@ MEASURED_BWD_TRAFFIC_BYTES = {
 }
 
 
+# Kernel names (as rocprofv3 prints them) of the dominant forward kernels, by the library's own name for the path
+_TRAFFIC_KERNELS = {"fwd_tile_f16": "fwd_h16_tile_kernel", "fwd_tile_bf16": "fwd_h16_tile_kernel", "fwd_tile_f32": "fwd_tile_kernel",
+                    "fwd_tiled_": "fwd_h16_kernel"}
+
+
+def _measure_traffic(argv_tail, kernel_hint, timeout_s=150):
+    """HBM-side bytes per launch of the dominant forward kernel, measured now: two child runs of this script under
+    `rocprofv3 --pmc` (FETCH_SIZE, then WRITE_SIZE: KiB per dispatch), each reading scaled by what the same counter
+    reads for a device copy of known size in the same run (`--calibrate-copy`: 64 MiB per dispatch).  Returns a dict,
+    or None when anything fails (no rocprofv3, counters refused, time-out): the caller then reports the recorded figure.
+    Runs before this process touches the GPU."""
+    import csv, glob, shutil, signal, subprocess, tempfile
+    rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(rocprof):
+        return None
+    here = os.path.abspath(__file__)
+    got = {}
+    tmp = tempfile.mkdtemp(prefix="ma_traffic_", dir="/tmp")
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            out = os.path.join(tmp, counter)
+            cmd = [rocprof, "--pmc", counter, "--kernel-trace", "-d", out, "--output-format", "csv", "--",
+                   sys.executable, here, "--no-cpu", "--no-extra", "--no-traffic", "--steps", "5", "--warmup", "2",
+                   "--calibrate-copy"] + argv_tail
+            env = dict(os.environ, TMPDIR="/tmp")
+            proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                                    start_new_session=True)
+            try:
+                if proc.wait(timeout=timeout_s) != 0:
+                    return None
+            except subprocess.TimeoutExpired:
+                os.killpg(proc.pid, signal.SIGKILL)
+                proc.wait()
+                return None
+            files = glob.glob(os.path.join(out, "**", "*counter_collection.csv"), recursive=True)
+            if not files:
+                return None
+            vals = {"kernel": [], "copy": []}
+            for row in csv.DictReader(open(files[0])):
+                if row.get("Counter_Name") != counter:
+                    continue
+                name = row.get("Kernel_Name", "")
+                if kernel_hint in name:
+                    vals["kernel"].append(float(row["Counter_Value"]))
+                elif "copyBuffer" in name:
+                    vals["copy"].append(float(row["Counter_Value"]))
+            if not vals["kernel"] or not vals["copy"]:
+                return None
+            got[counter] = (sum(vals["kernel"]) / len(vals["kernel"]), sum(vals["copy"]) / len(vals["copy"]), len(vals["kernel"]))
+    except Exception:
+        return None
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    copy_kib = 65536.0                                  # one copy dispatch: 64 MiB read, 64 MiB written
+    f_fetch, f_write = copy_kib / got["FETCH_SIZE"][1], copy_kib / got["WRITE_SIZE"][1]
+    if not (0.5 < f_fetch < 8 and 0.5 < f_write < 8):
+        return None
+    nbytes = (got["FETCH_SIZE"][0] * f_fetch + got["WRITE_SIZE"][0] * f_write) * 1024.0
+    return {"bytes": int(round(nbytes)), "fetch_kib": got["FETCH_SIZE"][0], "write_kib": got["WRITE_SIZE"][0],
+            "fetch_factor": f_fetch, "write_factor": f_write, "dispatches": got["FETCH_SIZE"][2]}
+
+
 def _events_ms(fn, steps, warmup):
     import torch
     for _ in range(warmup):
@@ -314,6 +376,9 @@ def main():
                          "line; for profiling); with HxW, e.g. 720x1280, only that size with the fused module step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="do not measure roofline.traffic in this run (two child runs under rocprofv3 --pmc, about a "
+                         "minute); the figure recorded in profiles/ is reported instead")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known HBM traffic, "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -322,6 +387,15 @@ def main():
         print("bench.py: this operator benchmark runs on exactly one GPU (--gpus 1); "
               "sharding across GPUs is a design note, not part of this build", file=sys.stderr)
         sys.exit(2)
+
+    # roofline.traffic of the headline line is measured by this run itself, before this process touches the GPU
+    traffic_now = None
+    if not (args.no_traffic or args.backward or args.e2e):
+        from matchattention_amd.workloads import WORKLOADS as _W
+        dt_name = args.dtype or {"float16": "f16", "float32": "f32", "bfloat16": "bf16"}[str(_W[args.workload].dtype).split(".")[-1]]
+        hint = "fwd_h16_kernel" if (args.direct and dt_name == "f16") else ("fwd_tiled_kernel" if args.direct else _TRAFFIC_KERNELS["fwd_tile_" + dt_name])
+        tail = ["--workload", args.workload] + (["--dtype", args.dtype] if args.dtype else []) + (["--direct"] if args.direct else [])
+        traffic_now = _measure_traffic(tail, hint)
 
     import torch
     from matchattention_amd import _cabi
@@ -392,6 +466,13 @@ def main():
     achieved = whole_call if dom_ms is None else alg_bytes / (dom_ms * 1e-3) / 1e9
     traffic = next((v for (w, k), v in MEASURED_TRAFFIC_BYTES.items()
                     if w == args.workload and kernel.startswith(k + "_")), None)
+    traffic_source = "recorded: profiles/ (rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE of an earlier run)" if traffic else None
+    if traffic_now is not None:
+        traffic = traffic_now["bytes"]
+        traffic_source = ("measured in this run: rocprofv3 --pmc, FETCH_SIZE %.0f KiB x %.3f + WRITE_SIZE %.0f KiB x %.3f per launch "
+                          "(factors from a 64 MiB device copy in the same runs; mean of %d launches)"
+                          % (traffic_now["fetch_kib"], traffic_now["fetch_factor"], traffic_now["write_kib"],
+                             traffic_now["write_factor"], traffic_now["dispatches"]))
 
     extra = {}
     if not args.no_extra:
@@ -566,6 +647,7 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic,
+            "traffic_source": traffic_source,
             "algorithmic_bytes_per_launch": alg_bytes,
             "dominant_kernel": kernel,
             "dominant_kernel_ms": dom_ms,
