@@ -309,6 +309,10 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
     // 6x6 window, 1.1x to 4.7x from 2^18 with the 4x4 window (at 2^17 the stereo field loses 18 %).
     const long long nhq = (long long)B * H * W * h;
     if (dtype == MATCHATTN_F32 && CH == 64) return nhq >= (rx == 2 ? (1ll << 17) : (1ll << 18));
+    // fp16 heads of 64 channels (half the head-queries per byte of the 32-channel shapes): 1.16x to 2x from 2^18
+    // head-queries with the 6x6 window (0.66x to 1.2x at 2^17), 1.2x to 2.1x from 2^19 with the 4x4 window (0.9x to
+    // 1.4x at 2^18).
+    if (dtype == MATCHATTN_F16 && CH == 64) return nhq >= (rx == 2 ? (1ll << 18) : (1ll << 19));
     const bool mat16 = dtype != MATCHATTN_F32 && CH == 32;        // fwd_h16_tile_kernel with its matrix-unit phases
     if (rx == 2) return nhq >= (dtype == MATCHATTN_F32 ? (1ll << 18) : mat16 ? (1ll << 19) : dtype == MATCHATTN_F16 ? (1ll << 20) : (1ll << 21));
     if (mat16 && dtype == MATCHATTN_F16) return nhq >= (1ll << 20);
