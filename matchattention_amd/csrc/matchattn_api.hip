@@ -247,7 +247,11 @@ void launch_sort(const ma::SortArgs &S, const SortLayout &sl, long long L, int h
         else if (S.dtype == MATCHATTN_F16) hipLaunchKernelGGL(ma::sort_probe_kernel<1>, pg, dim3(256), 0, s, S);
         else hipLaunchKernelGGL(ma::sort_probe_kernel<2>, pg, dim3(256), 0, s, S);
     }
-    hipLaunchKernelGGL(ma::sort_count_kernel, dim3((unsigned)((L + 256 * ma::kCountPerThread - 1) / (256 * ma::kCountPerThread)), (unsigned)(shared_known ? 1 : h)),
+    // (grid.x a multiple of the 8 XCDs, workgroup ids being dealt to them round-robin: the workgroups that count the
+    // same pixels for the other heads -- one grid row each -- then run on the same XCD and find the lines of positions,
+    // which hold all heads of a pixel side by side, in its L2; the workgroups past the map leave at once)
+    const unsigned count_blocks = (unsigned)((L + 256 * ma::kCountPerThread - 1) / (256 * ma::kCountPerThread));
+    hipLaunchKernelGGL(ma::sort_count_kernel, dim3((count_blocks + 7u) / 8u * 8u, (unsigned)(shared_known ? 1 : h)),
                        dim3(256), 0, s, S);
     hipLaunchKernelGGL(ma::sort_rowscan_kernel, dim3((unsigned)sl.nrows, (unsigned)h), dim3(64), 0, s, S);
     hipLaunchKernelGGL(ma::sort_rowtot_scan_kernel, dim3((unsigned)h), dim3(1024), 0, s, S);
