@@ -154,18 +154,19 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
  *                            1/2 tiled kernel with that many 16-byte vectors per lane
  *   name "stereo_row_skip":   1 (default) skip the last window row when every lane of a
  *                            wavefront has an integer y (its weights are exactly 0), 0 never
- *   name "forward_lds":      -1 (default) auto, 1 always, 0 never: r <= 2, head size 16/32/64 (fp16, bf16) or
- *                            16/32 (fp32), workspace given --
+ *   name "forward_lds":      -1 (default) auto, 1 always, 0 never: r <= 2, head size 16/32/64, workspace given --
  *                            bucket the queries by the 16x8 tile of K/V their window centre falls in, stage
  *                            each tile with its halo in LDS once and read every tap from LDS.  Auto uses it
- *                            for r = 2 from 2^20 head-queries (fp32: 2^18, bf16: 2^21) and for r = 1 from 2^21
- *                            (not in bf16).
+ *                            from the map sizes at which it measured faster than the direct kernel: with
+ *                            r = 2 from 2^19 head-queries for 32 fp16 or bf16 channels per head, 2^18 for 64
+ *                            fp16 channels, 2^20 for 16, 2^18 in fp32 (2^17 for 64 channels), 2^21 for the
+ *                            other bf16 head sizes; with r = 1 from 2^20 (fp16, 32 channels), 2^19 (fp16, 64),
+ *                            2^18 (fp32, 64), 2^21 otherwise (not for 16 or 64 bf16 channels).
  *   name "backward_mode":     -1 auto (default: gather where a tiled kernel exists), 0 scatter dK/dV with
  *                            fp32 atomics, 1 / 2 gather them per key through an inverse index
  *                            (deterministic) with the per-query pass on LDS tiles wherever that kernel
- *                            exists (1: head size 16/32/64 in fp16 and bf16, 16/32 in fp32) or always on the
- *                            direct kernel (2); auto
- *                            takes the tiles from 2^18 head-queries
+ *                            exists (1: head size 16/32/64) or always on the direct kernel (2); auto
+ *                            takes the tiles from 2^18 head-queries (2^17 for 64 fp32 channels per head)
  *   name "time_kernels":      0 (default) / 1: see matchattn_last_forward_kernel_ms
  *   name "xcd_swizzle":       1 (default) give each XCD a contiguous band of the image, 0 keep
  *                            the hardware's round-robin workgroup order
