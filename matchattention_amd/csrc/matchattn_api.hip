@@ -237,15 +237,25 @@ TileLayout tile_layout(int B, int H, int W, int h, bool by_row) {
 // zeroed flags already say "shared".
 void launch_sort(const ma::SortArgs &S, const SortLayout &sl, long long L, int h, char *ws, bool bin_order, hipStream_t s,
                  bool shared_known = false) {
-    const size_t nzero = sl.rowtot_off / 4;            // flags + counters
+    // Small maps, exact index: one workgroup per image and head builds it whole (the counters need no zeroing then)
+    const bool small = bin_order && S.force && S.bin_w == 1 && S.bin_h == 1 && S.sub_h == 1 && !S.pop && !S.shared_perm &&
+                       S.N <= ma::kSmallSortMaxN && S.W < 65536 && S.H < 65536;
+    const size_t nzero = small ? (size_t)ma::kFlagWords : sl.rowtot_off / 4;            // flags (+ counters)
     const size_t zb = nzero / 4 / 256 + 1;
-    shared_known = shared_known && S.force;
+    shared_known = (shared_known && S.force) || (small && h == 1);
     hipLaunchKernelGGL(ma::fill_zero_kernel, dim3((unsigned)(zb < 8192 ? zb : 8192)), dim3(256), 0, s, (float *)ws, nzero);
     if (!shared_known) {
         const dim3 pg((unsigned)std::min<long long>((L * h + 255) / 256, ma::kProbeBlocks));
         if (S.dtype == MATCHATTN_F32) hipLaunchKernelGGL(ma::sort_probe_kernel<0>, pg, dim3(256), 0, s, S);
         else if (S.dtype == MATCHATTN_F16) hipLaunchKernelGGL(ma::sort_probe_kernel<1>, pg, dim3(256), 0, s, S);
         else hipLaunchKernelGGL(ma::sort_probe_kernel<2>, pg, dim3(256), 0, s, S);
+    }
+    if (small) {
+        const dim3 g((unsigned)(L / S.N), (unsigned)h), t(ma::kSmallSortThreads);
+        if (S.dtype == MATCHATTN_F32) hipLaunchKernelGGL(ma::sort_small_kernel<0>, g, t, 0, s, S);
+        else if (S.dtype == MATCHATTN_F16) hipLaunchKernelGGL(ma::sort_small_kernel<1>, g, t, 0, s, S);
+        else hipLaunchKernelGGL(ma::sort_small_kernel<2>, g, t, 0, s, S);
+        return;
     }
     // (grid.x a multiple of the 8 XCDs, workgroup ids being dealt to them round-robin: the workgroups that count the
     // same pixels for the other heads -- one grid row each -- then run on the same XCD and find the lines of positions,

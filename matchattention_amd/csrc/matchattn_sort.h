@@ -424,4 +424,88 @@ __global__ __launch_bounds__(256) void sort_big_bins_store_kernel(SortArgs S) {
     }
 }
 
+// Small maps: the exact inverse index (bins of one pixel, entries of a bin in ascending pixel order, centres) of one
+// image and head from ONE workgroup, in place of the count, scan, scatter and ordering kernels above -- at a few
+// thousand pixels each of those is a launch that lasts longer than its work.  The workgroup counts the image's bins
+// in LDS, scans them there, places the entries (in arrival order) in an LDS copy of the order, and every entry then
+// finds its final place by counting the entries of its bin with a smaller pixel index: the result does not depend on
+// the order of the atomics.  Bins with more than kMaxRankedBin entries keep the arrival order, as above.
+// Grid (batch items, heads); the workgroups of heads 1.. leave when the heads share head 0's index (the probe has
+// run).  Writes count, rowtot, perm and centre exactly as the kernels above leave them (rank is not used).
+// (Letting every workgroup do the probe's work itself -- read all positions of the call, so that all come to the same
+// answer without exchanging a word -- saves the zeroing and the probe launches, but one CU reads the positions at a
+// fraction of the chip's rate: measured equal at 2 x 48 x 48 x 4 heads, 12 us slower at 2 x 96 x 96 x 4.)
+constexpr int kSmallSortMaxN = 10240, kSmallSortThreads = 1024;
+template <int DT>
+__global__ __launch_bounds__(kSmallSortThreads) void sort_small_kernel(SortArgs S) {
+    __shared__ int tab[kSmallSortMaxN];              // bin counts, then bin starts
+    __shared__ uint16_t order[kSmallSortMaxN];       // pixel (within the image) at each position, arrival order
+    __shared__ int wave_tot[kSmallSortThreads / 64];
+    const int b = blockIdx.x, hd = blockIdx.y, N = S.N, tid = threadIdx.x;
+    if (hd > 0 && *S.per_head == 0) return;          // uniform over the workgroup
+    constexpr int PER = kSmallSortMaxN / kSmallSortThreads;
+    for (int i = tid; i < N; i += kSmallSortThreads) tab[i] = 0;
+    float x[PER], y[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const int p = min(tid + u * kSmallSortThreads, N - 1);
+        load_xy_as<DT>(S.mo, ((size_t)b * N + p) * S.h + hd, x[u], y[u]);
+    }
+    __syncthreads();
+    int bin[PER], arrival[PER], ctr[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const uint32_t cell = target_cell(S, x[u], y[u]);        // bins of one pixel: (row << 16) | column
+        bin[u] = (int)(cell >> 16) * S.W + (int)(cell & 0xffffu);
+        ctr[u] = pack_centre(x[u], y[u]);
+        arrival[u] = tid + u * kSmallSortThreads < N ? atomicAdd(&tab[bin[u]], 1) : 0;
+    }
+    __syncthreads();
+    // exclusive scan of the counts, in place: a run of bins per thread, the runs' totals over the wavefront and the
+    // wavefronts' totals through LDS
+    {
+        const int per = (N + kSmallSortThreads - 1) / kSmallSortThreads;
+        const int lo = min(tid * per, N), hi = min(lo + per, N);
+        int s = 0;
+        for (int i = lo; i < hi; ++i) s += tab[i];
+        int incl = s;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int v = __shfl_up(incl, d, 64);
+            if ((tid & 63) >= d) incl += v;
+        }
+        if ((tid & 63) == 63) wave_tot[tid >> 6] = incl;
+        __syncthreads();
+        int run = incl - s;
+        for (int w = 0; w < (tid >> 6); ++w) run += wave_tot[w];
+        for (int i = lo; i < hi; ++i) { const int v = tab[i]; tab[i] = run; run += v; }
+    }
+    __syncthreads();
+    int *const count = S.count + (size_t)hd * S.nbins + (size_t)b * N;
+    for (int i = tid; i < N; i += kSmallSortThreads) {
+        const int row = i / S.W;
+        count[i] = tab[i] - tab[row * S.W];
+        if (i == row * S.W) S.rowtot[hd * S.nrows + b * S.H + row] = b * N + tab[i];
+    }
+#pragma unroll
+    for (int u = 0; u < PER; ++u)
+        if (tid + u * kSmallSortThreads < N) order[tab[bin[u]] + arrival[u]] = (uint16_t)(tid + u * kSmallSortThreads);
+    __syncthreads();
+    int *const perm = S.perm + (size_t)hd * S.L + (size_t)b * N;
+    int *const centre = S.centre ? S.centre + (size_t)hd * S.L + (size_t)b * N : nullptr;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const int p = tid + u * kSmallSortThreads;
+        if (p >= N) continue;
+        const int lo = tab[bin[u]], n = (bin[u] + 1 < N ? tab[bin[u] + 1] : N) - lo;
+        int r = arrival[u];
+        if (n > 1 && n <= kMaxRankedBin) {
+            r = 0;
+            for (int j = 0; j < n; ++j) r += (int)order[lo + j] < p ? 1 : 0;
+        }
+        perm[lo + r] = b * N + p;
+        if (centre) centre[lo + r] = ctr[u];
+    }
+}
+
 }  // namespace ma

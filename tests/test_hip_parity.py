@@ -143,6 +143,27 @@ def test_lds_tile_backward_matches_autograd(hip_lib, dt, offs, per_head, clamp, 
         assert rel_err(a.cpu(), d.cpu().double()) <= TOL[dt], nm     # the two pass-A kernels agree
 
 
+@pytest.mark.parametrize("per_head", [True, False], ids=["per_head", "shared"])
+@pytest.mark.parametrize("shape", [(1, 100, 100), (1, 110, 100), (3, 30, 40)], ids=lambda s: "x".join(map(str, s)))
+def test_inverse_index_of_small_and_larger_maps(hip_lib, shape, per_head):
+    # The per-key pass follows an inverse index (which queries sample each pixel).  Maps of up to 10240 pixels get it
+    # from one workgroup per image and head, larger ones from the chain of count, scan, scatter and ordering kernels:
+    # a map on either side of that size and a batch of small ones, with unclamped offsets of which a good share lies
+    # outside the map, so that the bins along the border hold hundreds of entries.  Gradients against the oracle's,
+    # and a second call bit for bit (the order inside a bin must not depend on the order of the atomics).
+    B, H, W = shape
+    h, Ch, r = 2, 16, 1
+    mo, q, k, v = make_case(B, H, W, h, Ch, r, torch.float32, seed=313, offsets="mixed", clamp=False, per_head=per_head)
+    g = torch.Generator().manual_seed(17)
+    d_out = torch.randn(B, H * W, h * Ch, generator=g)
+    d_attn = torch.randn(B, H * W, h, 16, generator=g)
+    dev = _dev(mo, q, k, v)
+    got = hip_backward(hip_lib, *dev, H, W, r, 0.25, d_out.cuda(), d_attn.cuda())
+    again = hip_backward(hip_lib, *dev, H, W, r, 0.25, d_out.cuda(), d_attn.cuda())
+    assert all(torch.equal(a, b) for a, b in zip(got, again))
+    check_grads(got, mo, q, k, v, H, W, r, 0.25, d_out, d_attn, "inverse index bwd")
+
+
 def test_backward_without_attention_gradient(hip_lib):
     B, H, W, h, Ch, r = 1, 9, 10, 2, 32, 2
     mo, q, k, v = make_case(B, H, W, h, Ch, r, torch.float32, seed=5)
