@@ -166,7 +166,10 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
  *                            fp32 atomics, 1 / 2 gather them per key through an inverse index
  *                            (deterministic) with the per-query pass on LDS tiles wherever that kernel
  *                            exists (1: head size 16/32/64) or always on the direct kernel (2); auto
- *                            takes the tiles from 2^18 head-queries (2^17 for 64 fp32 channels per head)
+ *                            takes the tiles from the sizes at which the whole backward measured faster with
+ *                            them: fp32 from 2^18 head-queries with r = 2, 2^19 with r = 1, 2^17 for heads of
+ *                            64 channels; fp16 from 2^19 (2^18 for 64 channels and r = 2); bf16 from 2^20
+ *                            with r = 2 and 1.5 * 2^20 with r = 1 (64 channels: 2^19 and 2^20)
  *   name "time_kernels":      0 (default) / 1: see matchattn_last_forward_kernel_ms
  *   name "xcd_swizzle":       1 (default) give each XCD a contiguous band of the image, 0 keep
  *                            the hardware's round-robin workgroup order

@@ -650,9 +650,23 @@ bool bwd_tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx
           h % (head_bytes >= 128 ? 1 : 128 / head_bytes) == 0 &&
           (unsigned long long)B * H * W * h * M * pair_bytes(dtype) < 0xFFFFF000ull))
         return false;
-    // auto: maps large enough to pay for the bucketing (heads of 64 fp32 channels, twice the bytes per head-query: 1.1x to
-    // 1.4x at 2^17 already)
-    return mode == 1 || (long long)B * H * W * h >= ((dtype == MATCHATTN_F32 && CH == 64) ? (1ll << 17) : (1ll << 18));
+    if (mode == 1) return true;
+    // auto: maps large enough to pay for the second bucketing.  Whole backward with pass A on tiles against the direct
+    // pass A, heads of 16 and 32 channels, i.i.d. and smooth fields, shared and per-head offsets (one process):
+    //   fp16  6x6 window: 0.91x to 1.02x at 2^18 head-queries, 0.98x to 1.27x at 2^19, 1.06x to 1.42x at 2^20;
+    //         4x4 window: 0.85x to 0.93x at 2^18, 0.92x to 1.08x at 2^19, 0.97x to 1.22x at 2^20
+    //   fp32  6x6: 0.89x to 1.14x at 2^18, 1.00x to 1.25x at 2^19;  4x4: 0.82x to 0.93x at 2^18, 0.88x to 1.12x at 2^19
+    //   bf16  6x6: 0.80x to 0.90x at 2^18, 0.85x to 1.12x at 2^19, 0.93x to 1.28x at 2^20;
+    //         4x4: 0.82x to 0.97x at 2^19, 0.87x to 1.08x at 2^20, 0.92x to 1.27x at 2^21
+    // (the smooth per-head field is the low end everywhere: its gathers already hit L1).  Heads of 64 channels, twice
+    // the bytes per head-query, pay one step earlier: fp32 1.1x to 1.4x at 2^17; fp16 6x6 1.00x to 1.17x at 2^18, 4x4
+    // 0.89x to 1.00x at 2^18 and 1.00x to 1.17x at 2^19; bf16 6x6 0.88x to 1.01x at 2^18 and 0.99x to 1.10x at 2^19, 4x4
+    // 0.94x to 1.04x at 2^19 and 0.98x to 1.10x at 2^20.
+    const long long nhq = (long long)B * H * W * h;
+    if (dtype == MATCHATTN_F32) return nhq >= (CH == 64 ? (1ll << 17) : rx == 2 ? (1ll << 18) : (1ll << 19));
+    if (dtype == MATCHATTN_F16) return nhq >= (rx == 2 && CH == 64 ? (1ll << 18) : (1ll << 19));
+    if (CH == 64) return nhq >= (rx == 2 ? (1ll << 19) : (1ll << 20));
+    return nhq >= (rx == 2 ? (1ll << 20) : (3ll << 19));
 }
 BwdLayout bwd_gather_layout(const Options &O, int B, int H, int W, int C, int h, int rx, int dtype) {
     BwdLayout l;
