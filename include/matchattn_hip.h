@@ -157,11 +157,12 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
  *   name "forward_lds":      -1 (default) auto, 1 always, 0 never: r <= 2, head size 16/32/64, workspace given --
  *                            bucket the queries by the 16x8 tile of K/V their window centre falls in, stage
  *                            each tile with its halo in LDS once and read every tap from LDS.  Auto uses it
- *                            from the map sizes at which it measured faster than the direct kernel: with
- *                            r = 2 from 2^19 head-queries for 32 fp16 or bf16 channels per head, 2^18 for 64
- *                            fp16 channels, 2^20 for 16, 2^18 in fp32 (2^17 for 64 channels), 2^21 for the
- *                            other bf16 head sizes; with r = 1 from 2^20 (fp16, 32 channels), 2^19 (fp16, 64),
- *                            2^18 (fp32, 64), 2^21 otherwise (not for 16 or 64 bf16 channels).
+ *                            from the map sizes at which it measured faster than the direct kernel over
+ *                            i.i.d. and smooth offset fields (geometric mean), in head-queries B*H*W*h:
+ *                              fp16  r = 2: 2^20 (32 channels per head), 2^19 (64), 1.5 * 2^20 (16);
+ *                                    r = 1: 2^21 (32 and 16), 2^20 (64)
+ *                              bf16  r = 2: 2^20 (32 and 64), 2^21 (16); r = 1: 2^21 (32), never (16, 64)
+ *                              fp32  r = 2: 2^19 (16 and 32), 2^17 (64); r = 1: 2^20 (32), 1.5 * 2^20 (16), 2^18 (64)
  *   name "backward_mode":     -1 auto (default: gather where a tiled kernel exists), 0 scatter dK/dV with
  *                            fp32 atomics, 1 / 2 gather them per key through an inverse index
  *                            (deterministic) with the per-query pass on LDS tiles wherever that kernel

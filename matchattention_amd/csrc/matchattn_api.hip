@@ -310,27 +310,38 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
     if (!(CH == 16 || CH == 32 || CH == 64)) return false;
     if (h % (head_bytes >= 128 ? 1 : 128 / head_bytes) != 0) return false;
     if (mode == 1) return true;
-    // auto: sizes that fill the chip.  Measured against the direct gather (stereo, per-head and 2-D random fields, 8 and
-    // 16 heads, one process): with the 6x6 window the tiles win from about 2^19 head-queries with 32 16-bit channels per
-    // head (the kernel that uses the matrix unit; fp16 1.3x to 2.2x at 2^19, 0.75x to 1.3x at 2^18; bf16 1.1x to 2.2x and
-    // 0.9x to 1.7x), from 2^20 with the other fp16 head sizes, from 2^18 in fp32 (whose direct kernel moves twice the
-    // bytes through L2: 1.1x to 4x) and from 2^21 with the other bf16 head sizes (at 2^20 the stereo field still loses
-    // 10 %); with the 4x4 window from 2^20 in fp16 with 32 channels per head (1.07x to 1.9x; at 2^19 the stereo field
-    // loses 13 %), from about 2^21 with the other fp16 head sizes, in fp32 and in bf16 with 32 channels per head (1.5x to
-    // 2x on per-head and 2-D fields; the bf16 stereo field loses 4 % there), and with the other bf16 head sizes only on
-    // incoherent fields, so not by default.  Below that bucketing the queries costs more than it saves.
-    // Heads of 64 fp32 channels (one workgroup of 512 threads per CU): 1.3x to 5.8x from 2^17 head-queries with the
-    // 6x6 window, 1.1x to 4.7x from 2^18 with the 4x4 window (at 2^17 the stereo field loses 18 %).
-    const long long nhq = (long long)B * H * W * h;
-    if (dtype == MATCHATTN_F32 && CH == 64) return nhq >= (rx == 2 ? (1ll << 17) : (1ll << 18));
-    // fp16 heads of 64 channels (half the head-queries per byte of the 32-channel shapes): 1.16x to 2x from 2^18
-    // head-queries with the 6x6 window (0.66x to 1.2x at 2^17), 1.2x to 2.1x from 2^19 with the 4x4 window (0.9x to
-    // 1.4x at 2^18).
-    if (dtype == MATCHATTN_F16 && CH == 64) return nhq >= (rx == 2 ? (1ll << 18) : (1ll << 19));
-    const bool mat16 = dtype != MATCHATTN_F32 && CH == 32;        // fwd_h16_tile_kernel with its matrix-unit phases
-    if (rx == 2) return nhq >= (dtype == MATCHATTN_F32 ? (1ll << 18) : mat16 ? (1ll << 19) : dtype == MATCHATTN_F16 ? (1ll << 20) : (1ll << 21));
-    if (mat16 && dtype == MATCHATTN_F16) return nhq >= (1ll << 20);
-    return (dtype != MATCHATTN_BF16 || mat16) && nhq >= (1ll << 21);
+    // auto: the sizes from which the tiles win.  Measured against the direct gather in one process on five fields per
+    // size -- i.i.d. stereo (x - U(0, W/4), y exact), i.i.d. per-head 2-D (sigma 8), and three smooth ones as a model
+    // produces them (blurred stereo, a synthetic scene's disparity, blurred per-head) -- with 4 and 8 heads, 2^18 to
+    // 2^22 head-queries; the limit is where the geometric mean over the five crosses 1.  The smooth fields decide it:
+    // their gathers hit L1 and L2 and the direct kernel needs no bucketing, so the tiles win later than on the i.i.d.
+    // fields (and on the i.i.d. 2-D field they win 1.2x to 2x already one step below every limit given here).
+    //   fp16, 32 channels per head (the kernel with the matrix-unit phases):
+    //     6x6 window: 0.71x to 1.29x at 2^19, 1.16x to 2.1x at 2^20, 1.28x to 2.7x at 2^21, 1.43x to 3.2x at 2^22
+    //     4x4 window: 0.68x to 1.36x at 2^20, 0.77x to 1.78x at 2^21 (mean 1.0), 0.87x to 2.2x at 2^22
+    //   fp16, 64 channels: 6x6 0.66x to 0.81x at 2^18, 0.99x to 1.33x at 2^19; 4x4 0.78x to 1.13x at 2^19, 0.89x to
+    //     1.56x at 2^20;  16 channels: 6x6 0.66x to 1.94x at 2^20 (mean 0.86), 1.05x to 3.0x at 2^21; 4x4 not below 2^21
+    //   bf16, 32 channels: 6x6 0.78x to 1.48x at 2^19 (mean 0.95), 1.05x to 2.45x at 2^20; 4x4 0.73x to 1.9x at 2^20,
+    //     0.86x to 2.2x at 2^21 (mean 1.07);  64 channels: 6x6 0.87x to 1.26x at 2^19, 1.0x to 1.53x at 2^20; 4x4 and
+    //     16 channels: only the i.i.d. 2-D field wins below 2^21 (6x6 from 2^21, 4x4 not by default)
+    //   fp32 (whose direct kernel moves twice the bytes through L2), 16 and 32 channels: 6x6 0.61x to 1.24x at 2^18,
+    //     0.84x to 2.1x at 2^19 (mean 1.03 and 1.4); 4x4 32 channels 0.79x to 1.46x at 2^19, 0.91x to 2.1x at 2^20, 16
+    //     channels 0.80x to 1.31x at 2^20, 0.95x to 2.5x at 2^21;  64 channels (one workgroup of 512 threads per CU):
+    //     6x6 1.3x to 2.3x at 2^18, 4x4 0.88x to 1.62x at 2^18 (mean 1.03), 1.01x to 2.4x at 2^19
+    const long long nhq = (long long)B * H * W * h, k19 = 1ll << 19, k20 = 1ll << 20, k21 = 1ll << 21;
+    if (dtype == MATCHATTN_F32) {
+        if (CH == 64) return nhq >= (rx == 2 ? (1ll << 17) : (1ll << 18));
+        if (rx == 2) return nhq >= k19;
+        return nhq >= (CH == 32 ? k20 : k20 + k19);
+    }
+    if (dtype == MATCHATTN_F16) {
+        if (CH == 64) return nhq >= (rx == 2 ? k19 : k20);
+        if (CH == 32) return nhq >= (rx == 2 ? k20 : k21);
+        return nhq >= (rx == 2 ? k20 + k19 : k21);
+    }
+    if (CH == 32) return nhq >= (rx == 2 ? k20 : k21);
+    if (CH == 64) return rx == 2 && nhq >= k20;
+    return rx == 2 && nhq >= k21;
 }
 }  // namespace
 
