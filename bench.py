@@ -391,7 +391,8 @@ def main():
     # roofline.traffic of the headline line is measured by this run itself, before this process touches the GPU
     traffic_now = None
     if not (args.no_traffic or args.backward or args.e2e):
-        from matchattention_amd.workloads import WORKLOADS as _W
+        from matchattention_amd.workloads import WORKLOADS as _W0, MODEL_SHAPES as _W1
+        _W = {**_W0, **_W1}
         dt_name = args.dtype or {"float16": "f16", "float32": "f32", "bfloat16": "bf16"}[str(_W[args.workload].dtype).split(".")[-1]]
         hint = "fwd_h16_kernel" if (args.direct and dt_name == "f16") else ("fwd_tiled_kernel" if args.direct else _TRAFFIC_KERNELS["fwd_tile_" + dt_name])
         tail = ["--workload", args.workload] + (["--dtype", args.dtype] if args.dtype else []) + (["--direct"] if args.direct else [])
@@ -418,8 +419,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    wl = WORKLOADS[args.workload]
-    inp = make_inputs(wl)
+    # (--workload also takes the names of workloads.MODEL_SHAPES, the model's own operator shapes, on their smooth fields)
+    from matchattention_amd.workloads import MODEL_SHAPES
+    wl = WORKLOADS[args.workload] if args.workload in WORKLOADS else MODEL_SHAPES[args.workload]
+    inp = make_inputs(wl, smooth=args.workload in MODEL_SHAPES)
     if args.dtype:      # the same workload (same offset field and values, rounded) in another storage type
         import dataclasses
         dt = {"f16": torch.float16, "f32": torch.float32, "bf16": torch.bfloat16}[args.dtype]
