@@ -434,7 +434,10 @@ __global__ __launch_bounds__(256) void sort_big_bins_store_kernel(SortArgs S) {
 // run).  Writes count, rowtot, perm and centre exactly as the kernels above leave them (rank is not used).
 // (Letting every workgroup do the probe's work itself -- read all positions of the call, so that all come to the same
 // answer without exchanging a word -- saves the zeroing and the probe launches, but one CU reads the positions at a
-// fraction of the chip's rate: measured equal at 2 x 48 x 48 x 4 heads, 12 us slower at 2 x 96 x 96 x 4.)
+// fraction of the chip's rate: measured equal at 2 x 48 x 48 x 4 heads, 12 us slower at 2 x 96 x 96 x 4.  And the
+// limit is where one CU stops being faster than seven launches over the whole chip: a variant for images of up to
+// 40 448 pixels -- 16-bit counters, two per LDS word, the positions read three times -- took 90 us at 2 x 192 x 192
+// where the kernels above take 43.)
 constexpr int kSmallSortMaxN = 10240, kSmallSortThreads = 1024;
 template <int DT>
 __global__ __launch_bounds__(kSmallSortThreads) void sort_small_kernel(SortArgs S) {
