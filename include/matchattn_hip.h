@@ -161,7 +161,7 @@ int matchattn_backward(const void *max_offset, const void *q, const void *k, con
  *                            i.i.d. and smooth offset fields (geometric mean), in head-queries B*H*W*h:
  *                              fp16  r = 2: 2^20 (32 channels per head), 2^19 (64), 1.5 * 2^20 (16);
  *                                    r = 1: 2^21 (32 and 16), 2^20 (64)
- *                              bf16  r = 2: 2^20 (32 and 64), 2^21 (16); r = 1: 2^21 (32), never (16, 64)
+ *                              bf16  r = 2: 2^20 (32), 2^19 (64), 2^21 (16); r = 1: 2^21 (32), never (16, 64)
  *                              fp32  r = 2: 2^19 (16 and 32), 2^17 (64); r = 1: 2^20 (32), 1.5 * 2^20 (16), 2^18 (64)
  *   name "backward_mode":     -1 auto (default: gather where a tiled kernel exists), 0 scatter dK/dV with
  *                            fp32 atomics, 1 / 2 gather them per key through an inverse index

@@ -217,7 +217,10 @@ SortLayout sort_layout(int B, int H, int W, int h, int bin_w, int bin_h = 1, int
 struct TileLayout { SortLayout sl; size_t defer_off, chunk_off, item_off, total; int chunk_cap; };
 // `by_row`: the buckets are ordered by the window's row inside the tile (one sub-bucket per row), which the fp16
 // forward with 32 channels per head wants: its aggregation walks the rows the 16 queries of a wavefront reach.
-bool tile_rows_wanted(int C, int h, int dtype) { return (dtype == MATCHATTN_F16 || dtype == MATCHATTN_BF16) && C / h == 32; }
+bool tile_rows_wanted(int C, int h, int rx, int dtype) {
+    // (64 channels with the 6x6 window: as two half-heads of 32 on the same kernel)
+    return (dtype == MATCHATTN_F16 || dtype == MATCHATTN_BF16) && (C / h == 32 || (C / h == 64 && rx == 2));
+}
 TileLayout tile_layout(int B, int H, int W, int h, bool by_row) {
     TileLayout t;
     const int sub = by_row ? ma::kTileDims[1] : 1;
@@ -319,10 +322,10 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
     //   fp16, 32 channels per head (the kernel with the matrix-unit phases):
     //     6x6 window: 0.71x to 1.29x at 2^19, 1.16x to 2.1x at 2^20, 1.28x to 2.7x at 2^21, 1.43x to 3.2x at 2^22
     //     4x4 window: 0.68x to 1.36x at 2^20, 0.77x to 1.78x at 2^21 (mean 1.0), 0.87x to 2.2x at 2^22
-    //   fp16, 64 channels: 6x6 0.66x to 0.81x at 2^18, 0.99x to 1.33x at 2^19; 4x4 0.78x to 1.13x at 2^19, 0.89x to
+    //   fp16, 64 channels: 6x6 0.73x to 0.88x at 2^18, 1.13x to 1.50x at 2^19; 4x4 0.78x to 1.13x at 2^19, 0.89x to
     //     1.56x at 2^20;  16 channels: 6x6 0.66x to 1.94x at 2^20 (mean 0.86), 1.05x to 3.0x at 2^21; 4x4 not below 2^21
     //   bf16, 32 channels: 6x6 0.78x to 1.48x at 2^19 (mean 0.95), 1.05x to 2.45x at 2^20; 4x4 0.73x to 1.9x at 2^20,
-    //     0.86x to 2.2x at 2^21 (mean 1.07);  64 channels: 6x6 0.87x to 1.26x at 2^19, 1.0x to 1.53x at 2^20; 4x4 and
+    //     0.86x to 2.2x at 2^21 (mean 1.07);  64 channels: 6x6 0.89x to 1.04x at 2^18, 1.15x to 1.66x at 2^19; 4x4 and
     //     16 channels: only the i.i.d. 2-D field wins below 2^21 (6x6 from 2^21, 4x4 not by default)
     //   fp32 (whose direct kernel moves twice the bytes through L2), 16 and 32 channels: 6x6 0.61x to 1.24x at 2^18,
     //     0.84x to 2.1x at 2^19 (mean 1.03 and 1.4); 4x4 32 channels 0.79x to 1.46x at 2^19, 0.91x to 2.1x at 2^20, 16
@@ -340,7 +343,7 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
         return nhq >= (rx == 2 ? k20 + k19 : k21);
     }
     if (CH == 32) return nhq >= (rx == 2 ? k20 : k21);
-    if (CH == 64) return rx == 2 && nhq >= k20;
+    if (CH == 64) return rx == 2 && nhq >= k19;            // (as two half-heads of 32 on the same kernel: 1.15x to 1.66x at 2^19)
     return rx == 2 && nhq >= k21;
 }
 }  // namespace
@@ -348,7 +351,7 @@ bool tile_wanted(const Options &O, int B, int H, int W, int C, int h, int rx, in
 namespace {
 size_t forward_workspace_bytes(const Options &O, int B, int H, int W, int C, int h, int rx, int ry, int dtype) {
     if (B <= 0 || H <= 0 || W <= 0 || C <= 0 || h <= 0) return 0;
-    return tile_wanted(O, B, H, W, C, h, rx, ry, dtype) ? tile_layout(B, H, W, h, tile_rows_wanted(C, h, dtype)).total : 0;
+    return tile_wanted(O, B, H, W, C, h, rx, ry, dtype) ? tile_layout(B, H, W, h, tile_rows_wanted(C, h, rx, dtype)).total : 0;
 }
 }  // namespace
 
@@ -404,7 +407,7 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
         // LDS-tile path: bucket the queries by K/V tile, one workgroup per tile and head group, then the
         // generic kernel for the (normally empty) list of queries a tile could not serve
         if (workspace && P.rel_heads == 0 && tile_wanted(O, B, H, W, C, h, rx, ry, dtype) && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
-            const TileLayout tl = tile_layout(B, H, W, h, tile_rows_wanted(C, h, dtype));
+            const TileLayout tl = tile_layout(B, H, W, h, tile_rows_wanted(C, h, rx, dtype));
             const SortLayout &sl = tl.sl;
             if (workspace_bytes < tl.total)
                 return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_ws: workspace of %zu bytes needed, %zu given",
@@ -565,7 +568,7 @@ int matchattn_forward_deferred(const void *workspace, size_t workspace_bytes,
     if (!count) return fail(MATCHATTN_ERR_ARG, "matchattn_forward_deferred: null count pointer");
     *count = -1;
     if (!workspace || !tile_wanted(options_now(), B, H, W, C, h, rx, ry, dtype)) return MATCHATTN_OK;
-    const TileLayout tl = tile_layout(B, H, W, h, tile_rows_wanted(C, h, dtype));
+    const TileLayout tl = tile_layout(B, H, W, h, tile_rows_wanted(C, h, rx, dtype));
     if (workspace_bytes < tl.total)
         return fail(MATCHATTN_ERR_WORKSPACE, "matchattn_forward_deferred: workspace of %zu bytes needed, %zu given",
                     tl.total, workspace_bytes);

@@ -260,7 +260,12 @@ __global__ __launch_bounds__(1024) void tile_chunks_kernel(TileSort S, int h, in
 // halves (q is unpacked once per pass) and rounded to bf16 -- where the definition rounds them -- by the packed
 // conversion that feeds the matrix instruction; logits and weights are kept as packed bf16 pairs and unpacked by
 // shifts where the softmax needs them.
-template <int CH, int R, int TW, int TH, int VPL, typename T = half_t>
+// PAIRED: a head has 64 channels and is handled as two half-heads of 32 (CH = 32 here): the kernel's "heads" are then
+// the half-heads -- its head groups, 128 bytes per pixel, are the real heads -- whose L1 sums are added before anything is
+// rounded (the two half-heads of a query sit in neighbouring lanes: one cross-lane addition per tap), so that both hold
+// the head's logits, run the same softmax and aggregate their own 32 channels with the same weights on the matrix
+// unit.  Sampling position, bucket order, attention row and hand-over flag belong to the real head.
+template <int CH, int R, int TW, int TH, int VPL, typename T = half_t, bool PAIRED = false>
 __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(FwdArgs A, TileSort S) {
     constexpr bool kBf = std::is_same<T, bf16_t>::value;
     static_assert(kBf || std::is_same<T, half_t>::value, "16-bit storage types");
@@ -288,7 +293,8 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     static_assert(!kMatrixAgg || V_ZERO16 + 16 <= V_OFF + V_BYTES, "zeros for the lanes beyond a row");
     __shared__ __attribute__((aligned(16))) char smem[WM_OFF + WM_BYTES];   // K tile, V tile (+ zeros), weight rows
 
-    const int nhg = A.h / HPG;
+    static_assert(!PAIRED || (CH == 32 && HPG == 2 && VPL == 2), "a head of 64 channels as two half-heads of 32");
+    const int nhg = PAIRED ? A.h : A.h / HPG;
     const int npix = S.L;
     const uint32_t row_bytes = (uint32_t)A.C * 2u;
     const uint32_t total_bytes = (uint32_t)npix * row_bytes;
@@ -408,9 +414,10 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     const int hgrp = item_hgrp(item);
     const int bin = clampi(entry.x, 0, S.nbins - 1), part = max(entry.y, 0);
     // this lane group's head and its share of the bucket
-    const int head = hgrp * HPG + hslot;
+    const int head = hgrp * HPG + hslot;               // (PAIRED: the half-head, i.e. the block of 32 channels)
+    const int qhead = PAIRED ? hgrp : head;            // the head whose query this is: position, order, attention row, flag
     int lo, hi;
-    bucket_bounds(S, per_head ? head : 0, bin, lo, hi);
+    bucket_bounds(S, per_head ? qhead : 0, bin, lo, hi);
     const int row = bin / S.bins_per_row, tx = bin - row * S.bins_per_row;
     const int b = min(row / S.rows_per_img, npix / A.N - 1), ty = row - (row / S.rows_per_img) * S.rows_per_img;
     const int box_x = tx * TW - R, box_y = ty * TH - R;
@@ -420,7 +427,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     const uint32_t chan_bytes = (uint32_t)(head * CH + sub * 8) * 2u;      // vector u adds u * LPH * 16 bytes
 
     auto load_pix_raw = [&](int slot) __attribute__((always_inline)) {
-        return S.perm[(size_t)(per_head ? head : 0) * npix + min(slot, npix - 1)];
+        return S.perm[(size_t)(per_head ? qhead : 0) * npix + min(slot, npix - 1)];
     };
     auto load_pix = [&](int slot) __attribute__((always_inline)) { return clampi(load_pix_raw(slot), 0, npix - 1); };
 
@@ -450,7 +457,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     __builtin_amdgcn_sched_barrier(0);                // (the wait for the pixel indices comes after these loads)
     pix = clampi(pix, 0, npix - 1);
     pix_n = clampi(pix_n, 0, npix - 1);
-    uint32_t xyu = __builtin_amdgcn_raw_buffer_load_b32(rm, (int)((uint32_t)(pix * A.h + head) * 4u), 0, 0);
+    uint32_t xyu = __builtin_amdgcn_raw_buffer_load_b32(rm, (int)((uint32_t)(pix * A.h + qhead) * 4u), 0, 0);
     u32x4 qv[VPL];
 #pragma unroll
     for (int u = 0; u < VPL; ++u) qv[u] = buf_load16(rq, (uint32_t)pix * row_bytes + chan_bytes + vec_off[u]);
@@ -485,7 +492,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
     if (__builtin_amdgcn_ballot_w64(valid) != 0) do {
         // next pass: its pixel index is known, fetch its offset and q now; and the index after it
         const int pix_nn = load_pix(slot + 2 * QPP);
-        const uint32_t xyu_n = __builtin_amdgcn_raw_buffer_load_b32(rm, (int)((uint32_t)(pix_n * A.h + head) * 4u), 0, 0);
+        const uint32_t xyu_n = __builtin_amdgcn_raw_buffer_load_b32(rm, (int)((uint32_t)(pix_n * A.h + qhead) * 4u), 0, 0);
         u32x4 qv_n[VPL];
 #pragma unroll
         for (int u = 0; u < VPL; ++u) qv_n[u] = buf_load16(rq, (uint32_t)pix_n * row_bytes + chan_bytes + vec_off[u]);
@@ -493,7 +500,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
 #pragma unroll
         for (int u = 0; u < VPL; ++u) gatev[u] = buf_load16(rgate, (uint32_t)pix * row_bytes + chan_bytes + vec_off[u]);
 
-        const int hq = pix * A.h + head;
+        const int hq = pix * A.h + qhead;
         const float x = pair_lo(pair_of(xyu)), y = pair_hi(pair_of(xyu));
         float x0, y0, w[4];
         corner_weights<T>(x, y, x0, y0, w);
@@ -594,6 +601,11 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                     }
                     static_assert(!kMatrixSum || VPL == 2, "one result row per vector of a lane");
                     sum = acc4[0] + acc4[1];
+                    if constexpr (PAIRED) {
+                        // the other half-head's sum, from the neighbouring lane (DPP quad_perm [1, 0, 3, 2]): an addition
+                        // of two floats gives both lanes the same bits
+                        sum += dpp_mov<0xB1>(sum);
+                    }
                     if constexpr (!kMatrixAgg || j == WN - 1) finite_check += sum;
                 } else {
                     sum = l1_sum<T>(qv[0], buf[s & 1][t][0]);
@@ -815,7 +827,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 uint32_t dw[NDW];
 #pragma unroll
                 for (int m = 0; m < NDW; ++m) dw[m] = pair_bits(ap[m / HW][m % HW]);
-                const uint32_t a_row = mine ? (uint32_t)pix * A.attn_row_bytes + (uint32_t)head * (uint32_t)(M * 2) : kDeadOffset;
+                const uint32_t a_row = mine ? (uint32_t)pix * A.attn_row_bytes + (uint32_t)qhead * (uint32_t)(M * 2) : kDeadOffset;
 #pragma unroll
                 for (int t = 0; t * LPH < NP; ++t) {
                     u32x4 piece = u32x4{dw[0], dw[1], dw[2], dw[3]};
@@ -862,7 +874,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
             const int delta = cyv - cy_min;
             const int t_hi = min(spread, kMaxDelta) + WN - 1 - (drop_last ? 1 : 0);     // last row step with a weight in it
             const bool mine = valid && fits && !far;
-            store_attn(mine);
+            store_attn(mine && (!PAIRED || hslot == 0));   // (PAIRED: both half-heads hold the row; one writes it)
             char *const wm = smem + WM_OFF + (threadIdx.x >> 6) * WM_WAVE_BYTES;
             const int jcol = lane_w & 15, gblk = lane_w >> 4;
             // lane `sub` of a head-query writes the halves sub, 2 + sub, ... of a window row: kept in the low halves
@@ -965,6 +977,7 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
                 const unsigned long long bad_m = __builtin_amdgcn_ballot_w64((any & 0x80008000u) != 0u);
                 ok_o[hg] = mine_o[hg] != 0 && (bad_m & col) == 0;
             }
+            if constexpr (PAIRED) ok_o[0] = ok_o[1] = ok_o[0] && ok_o[1];     // one head-query: all 64 channels, or none
             if (A.gate) {
 #pragma unroll
                 for (int hg = 0; hg < HPG; ++hg) ov[hg] = vec_mul<T>(ov[hg], gate_o[hg]);
@@ -973,7 +986,8 @@ __global__ __launch_bounds__(kTileNT, MA_TILE_WAVES) void fwd_h16_tile_kernel(Fw
             for (int hg = 0; hg < HPG; ++hg) {
                 const int head_o = hgrp * HPG + hg;
                 // the flag of the head-query (its valid owner wrote nothing: one store per head-query, from block 0's lane)
-                __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(ok_o[hg] ? 0 : 1), rd, (valid_o[hg] && gblk == 0) ? pix_o[hg] * A.h + head_o : (int)kDeadOffset, 0, 0);
+                if (!PAIRED || hg == 0)
+                    __builtin_amdgcn_raw_buffer_store_b8((uint8_t)(ok_o[hg] ? 0 : 1), rd, (valid_o[hg] && gblk == 0) ? pix_o[hg] * A.h + (PAIRED ? hgrp : head_o) : (int)kDeadOffset, 0, 0);
                 buf_store16(ro, ok_o[hg] ? (uint32_t)pix_o[hg] * A.out_row_bytes + (uint32_t)(head_o * CH * 2 + gblk * 16) : kDeadOffset, ov[hg]);
             }
         } else {

@@ -16,13 +16,18 @@ void launch_tile_chunks(const TileSort &S, int h, int queries_per_pass, hipStrea
 template <int CH, int R>
 static int launch_tile(const FwdArgs &A, const TileSort &S, hipStream_t s) {
     constexpr int VPL = CH >= 8 * MA_TILE_VPL ? MA_TILE_VPL : 1;      // vectors per lane
-    typedef TileCfg<CH, R, kTileW, kTileH, VPL> Cfg;
-    if (A.h % Cfg::HPG != 0) return -1;
+    // (heads of 64 channels, 6x6 window: as two half-heads of 32 each on the kernel with the matrix-unit phases -- 1.06x
+    // to 1.14x faster than the instance for 64 channels; with the 4x4 window 0.84x to 0.89x, so not there)
+    constexpr bool kPaired = CH == 64 && R == 2 && MA_TILE_VPL == 2;
+    typedef TileCfg<kPaired ? 32 : CH, R, kTileW, kTileH, VPL> Cfg;
+    if (!kPaired && A.h % Cfg::HPG != 0) return -1;
     FwdArgs B = A;
     launch_tile_chunks(S, A.h, Cfg::QPP, s);
     // persistent grid: a multiple of the 8 XCDs; two workgroups fit a CU's LDS
     const unsigned grid = tile_grid(2u * (unsigned)kTileGridMult);
     timer_mark(false, s);
+    if constexpr (kPaired) hipLaunchKernelGGL((fwd_h16_tile_kernel<32, R, kTileW, kTileH, 2, half_t, true>), dim3(grid), dim3(kTileNT), 0, s, B, S);
+    else
     hipLaunchKernelGGL((fwd_h16_tile_kernel<CH, R, kTileW, kTileH, VPL>), dim3(grid), dim3(kTileNT), 0, s, B, S);
     timer_mark(true, s);
     return (int)hipGetLastError();

@@ -27,12 +27,19 @@ static int launch_tile(const FwdArgs &A, const TileSort &S, hipStream_t s) {
     constexpr int NT = CH * (int)sizeof(T) > 128 ? 2 * kTileNT : kTileNT;   // 256-byte heads: one workgroup of 512 per CU
     typedef TileCfgT<T, CH, R, kTileW, kTileH, VPL, NT> Cfg;
     if (A.h % Cfg::HPG != 0) return -1;
+#if MA_DTYPE == 2
+    // (64 bf16 channels per head, 6x6 window: as two half-heads of 32 each on the 16-bit kernel, 64 queries per head
+    // and pass -- 1.22x to 1.37x faster than this file's kernel; with the 4x4 window 0.95x to 1.02x, so not there)
+    launch_tile_chunks(S, A.h, CH == 64 && R == 2 ? 64 : Cfg::QPP, s);
+#else
     launch_tile_chunks(S, A.h, Cfg::QPP, s);
+#endif
     const unsigned grid = tile_grid((unsigned)Cfg::WG_PER_CU * (unsigned)kTileGridMult);   // persistent: what fits a CU's LDS
     timer_mark(false, s);
 #if MA_DTYPE == 2
     // 32 bf16 channels per head: the 16-bit kernel with its sums and its aggregation on the matrix unit
     if constexpr (CH == 32) hipLaunchKernelGGL((fwd_h16_tile_kernel<CH, R, kTileW, kTileH, 2, bf16_t>), dim3(grid), dim3(kTileNT), 0, s, A, S);
+    else if constexpr (CH == 64 && R == 2) hipLaunchKernelGGL((fwd_h16_tile_kernel<32, R, kTileW, kTileH, 2, bf16_t, true>), dim3(grid), dim3(kTileNT), 0, s, A, S);
     else
 #endif
     hipLaunchKernelGGL((fwd_tile_kernel<T, CH, R, kTileW, kTileH, VPL, NT>), dim3(grid), dim3(NT), 0, s, A, S);

@@ -700,15 +700,19 @@ def test_non_finite_offsets_stay_local(hip_lib, dt, lds, bmode):
     assert torch.isfinite(bad_f[0][0, finite_rows]).all() and torch.isfinite(bad_f[1][0, finite_rows]).all()
 
 
+@pytest.mark.parametrize("Ch", [32, 64])
 @pytest.mark.parametrize("dt,big", [(torch.float16, 6.0e4), (torch.bfloat16, 3.0e38)], ids=["f16", "bf16"])
-def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib, dt, big):
+def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib, dt, big, Ch):
     # The 16-bit LDS-tile kernel adds the |q - k| of a lane pair with a matrix instruction whose zero entries multiply the
     # values of the other head-queries of the wavefront: 0 * inf = NaN.  A non-finite q or k value (or a difference
     # that overflows: 6e4 - (-6e4) in fp16, 3e38 - (-3e38) in bf16) must only change the queries that own it or whose window reaches it.
+    # (Heads of 64 channels run on the same kernel as two half-heads of 32, whose sums meet before the softmax and whose
+    # outputs are checked together: the poisoned channels lie in either half, and V is poisoned as well -- the
+    # aggregation multiplies the V values of a whole row of the tile by the zeros of the queries that do not reach them.)
     from matchattention_amd import _cabi
-    B, H, W, h, Ch, r = 1, 40, 50, 4, 32, 2
+    B, H, W, h, r = 1, 40, 50, 4, 2
     mo, q, k, v = make_case(B, H, W, h, Ch, r, dt, seed=77, offsets="interior", per_head=False)
-    qb, kb = q.clone(), k.clone()
+    qb, kb, vb = q.clone(), k.clone(), v.clone()
     q_poison = {5 * W + 7: float("inf"), 17 * W + 30: float("nan"), 30 * W + 12: big}
     k_poison = {9 * W + 40: -float("inf"), 22 * W + 21: float("nan"), 33 * W + 5: -big}
     for n, val in q_poison.items():
@@ -716,6 +720,8 @@ def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib, dt, big):
         qb[0, n, Ch + 9] = val
     for n, val in k_poison.items():
         kb[0, n, 2 * Ch + 1] = val
+        vb[0, n, 3 * Ch - 3] = val                       # (head 2, its last channels)
+    qb[0, 5 * W + 7, Ch - 5] = float("nan")              # (head 0, its last channels)
     # the query of the large entry reaches keys that hold its negative in the same channel: the difference overflows
     kb[0, 30 * W + 12, 3] = -big
     k_bad = set(k_poison) | {30 * W + 12}
@@ -734,9 +740,9 @@ def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib, dt, big):
         _cabi.set_option("forward_lds", 1)
         good = hip_forward(hip_lib, *_dev(mo, q, k, v), H, W, r, 0.2)
         assert _cabi.last_forward_kernel().startswith("fwd_tile_f16" if dt == torch.float16 else "fwd_tile_bf16")
-        bad = hip_forward(hip_lib, *_dev(mo, qb, kb, v), H, W, r, 0.2)
+        bad = hip_forward(hip_lib, *_dev(mo, qb, kb, vb), H, W, r, 0.2)
         _cabi.set_option("forward_lds", 0)
-        direct = hip_forward(hip_lib, *_dev(mo, qb, kb, v), H, W, r, 0.2)
+        direct = hip_forward(hip_lib, *_dev(mo, qb, kb, vb), H, W, r, 0.2)
     finally:
         _cabi.set_option("forward_lds", -1)
     keep = ~touched.cuda()
@@ -756,7 +762,7 @@ def test_non_finite_values_stay_local_on_the_matrix_unit(hip_lib, dt, big):
             assert torch.equal(torch.isfinite(a[0, own]), torch.isfinite(b[0, own]))
         try:
             _cabi.set_option("forward_lds", 1)
-            bad = hip_forward(hip_lib, *_dev(mo, qb, kb, v), H, W, r, 0.2)
+            bad = hip_forward(hip_lib, *_dev(mo, qb, kb, vb), H, W, r, 0.2)
         finally:
             _cabi.set_option("forward_lds", -1)
 
