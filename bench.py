@@ -391,8 +391,8 @@ def main():
     # roofline.traffic of the headline line is measured by this run itself, before this process touches the GPU
     traffic_now = None
     if not (args.no_traffic or args.backward or args.e2e):
-        from matchattention_amd.workloads import WORKLOADS as _W0, MODEL_SHAPES as _W1
-        _W = {**_W0, **_W1}
+        from matchattention_amd.workloads import WORKLOADS as _W0, MODEL_SHAPES as _W1, MODEL_SHAPES_BASE_F32 as _W2
+        _W = {**_W0, **_W1, **_W2}
         dt_name = args.dtype or {"float16": "f16", "float32": "f32", "bfloat16": "bf16"}[str(_W[args.workload].dtype).split(".")[-1]]
         hint = "fwd_h16_kernel" if (args.direct and dt_name == "f16") else ("fwd_tiled_kernel" if args.direct else _TRAFFIC_KERNELS["fwd_tile_" + dt_name])
         tail = ["--workload", args.workload] + (["--dtype", args.dtype] if args.dtype else []) + (["--direct"] if args.direct else [])
@@ -420,9 +420,10 @@ def main():
         del src, dst
 
     # (--workload also takes the names of workloads.MODEL_SHAPES, the model's own operator shapes, on their smooth fields)
-    from matchattention_amd.workloads import MODEL_SHAPES
-    wl = WORKLOADS[args.workload] if args.workload in WORKLOADS else MODEL_SHAPES[args.workload]
-    inp = make_inputs(wl, smooth=args.workload in MODEL_SHAPES)
+    from matchattention_amd.workloads import MODEL_SHAPES, MODEL_SHAPES_BASE_F32
+    _models = {**MODEL_SHAPES, **MODEL_SHAPES_BASE_F32}
+    wl = WORKLOADS[args.workload] if args.workload in WORKLOADS else _models[args.workload]
+    inp = make_inputs(wl, smooth=args.workload in _models)
     if args.dtype:      # the same workload (same offset field and values, rounded) in another storage type
         import dataclasses
         dt = {"f16": torch.float16, "f32": torch.float32, "bf16": torch.bfloat16}[args.dtype]
@@ -584,9 +585,10 @@ def main():
             torch.cuda.empty_cache()
         # the operator at the shapes a MatchStereo-T frame calls it with (1536 x 1536 input: maps of 48^2 .. 384^2, B = 2),
         # forward and backward, on smooth fields: mostly one launch of a few microseconds, bound by launch latency
-        from matchattention_amd.workloads import MODEL_SHAPES
+        # (and at the `base` variant's in fp32, the script's default precision: heads of up to 128 fp32 channels)
+        from matchattention_amd.workloads import MODEL_SHAPES, MODEL_SHAPES_BASE_F32
         shapes = {}
-        for name, w6 in MODEL_SHAPES.items():
+        for name, w6 in list(MODEL_SHAPES.items()) + list(MODEL_SHAPES_BASE_F32.items()):
             i6 = make_inputs(w6, smooth=True)
             rec = {}
             c8, k8 = _forward_call(lib, w6, i6)
@@ -603,7 +605,8 @@ def main():
             rec["bwd_kernel"] = _cabi.last_backward_kernel()
             shapes[name] = rec
             del k8, k9, i6
-        extra["model_shapes_matchstereo_tiny_1536"] = shapes
+        extra["model_shapes_matchstereo_tiny_1536"] = {k_: v_ for k_, v_ in shapes.items() if k_ in MODEL_SHAPES}
+        extra["model_shapes_matchstereo_base_fp32_1536"] = {k_: v_ for k_, v_ in shapes.items() if k_ in MODEL_SHAPES_BASE_F32}
         torch.cuda.empty_cache()
         # a plain device-to-device copy on this box, read + write bytes per second (what the HBM path delivers
         # to the simplest possible kernel)

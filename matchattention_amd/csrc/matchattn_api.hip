@@ -150,7 +150,7 @@ bool tiled_ok(const void *const *ptrs, int nptr, long long L, int C, int CH, int
 
 bool bwd_tiled_shape(int CH, int rx, int dtype) {
     if (rx > 2) return false;
-    const int f16set[] = {8, 16, 32, 40, 64, 80, 128}, f32set[] = {8, 16, 32, 40, 64};
+    const int f16set[] = {8, 16, 32, 40, 64, 80, 96, 128, 192}, f32set[] = {8, 16, 32, 40, 64, 80, 96, 128, 192};
     if (dtype == MATCHATTN_F32) { for (int c : f32set) if (c == CH) return true; return false; }
     for (int c : f16set) if (c == CH) return true;
     return false;
@@ -442,10 +442,15 @@ int forward_impl(const Options &O, const void *max_offset, const void *q, const 
                             hipGetErrorString((hipError_t)rc));
         }
         ma::timer_mark(false, s);
-        switch (dtype) {
-        case MATCHATTN_F32: rc = ma::launch_fwd_tiled_f32(A, CH, rx, vpl, s, &kname); break;
-        case MATCHATTN_F16: rc = ma::launch_fwd_tiled_f16(A, CH, rx, vpl, s, &kname); break;
-        default: rc = ma::launch_fwd_tiled_bf16(A, CH, rx, vpl, s, &kname); break;
+        // (auto: one vector per lane; head sizes of more than 16 vectors -- 80, 96, 128 fp32 channels, 192 in the 16-bit
+        // types -- only exist with two)
+        for (int v = vpl; v <= (variant > 0 ? vpl : 2); ++v) {
+            switch (dtype) {
+            case MATCHATTN_F32: rc = ma::launch_fwd_tiled_f32(A, CH, rx, v, s, &kname); break;
+            case MATCHATTN_F16: rc = ma::launch_fwd_tiled_f16(A, CH, rx, v, s, &kname); break;
+            default: rc = ma::launch_fwd_tiled_bf16(A, CH, rx, v, s, &kname); break;
+            }
+            if (rc != -1) break;
         }
         ma::timer_mark(true, s);
         if (rc == -1 && variant > 0)

@@ -30,7 +30,8 @@ __device__ __forceinline__ void tap_interval(int c, int key, int n, int R, int W
 // 5 waves per SIMD, two at 128 and 4.  Measured (fp16, 32 channels per head, 6x6 window): one vector is 1 % faster
 // with a shared offset and 1.5 % faster with per-head offsets; with the 4x4 window 10 %.  Squeezing the registers
 // further (6 or 8 waves) spills.
-template <typename T, int CH, int R> struct KeyVpl { static constexpr int value = 1; };
+// (heads of more than 16 vectors -- 80, 96, 128 fp32 channels, 192 in the 16-bit types -- take two per lane)
+template <typename T, int CH, int R> struct KeyVpl { static constexpr int value = CH * (int)sizeof(T) > 256 ? 2 : 1; };
 
 // COMPACT (maps below 2^25 pixels whose pair array stays below 4 GiB: chosen by the host): away from the border a
 // prepared candidate travels as one word, (query pixel << 6) | tap, or -1 for none -- one lane exchange instead of two

@@ -47,9 +47,8 @@ static int launch_tiled(const BwdArgs &A, hipStream_t s) {
 
 int MA_CAT(launch_bwd_tiled_, MA_SUFFIX)(const BwdArgs &A, int CH, int R, hipStream_t s, const char **name) {
     MA_CASE(8) MA_CASE(16) MA_CASE(32) MA_CASE(40) MA_CASE(64)
-#if MA_DTYPE != 0
-    MA_CASE(80) MA_CASE(128)
-#endif
+    // (the coarse levels of the reference's larger variants; beyond 16 vectors per head a head-query takes 32 lanes)
+    MA_CASE(80) MA_CASE(96) MA_CASE(128) MA_CASE(192)
     (void)A; (void)s; (void)name;
     return -1;
 }
@@ -73,9 +72,7 @@ static int launch_key(const BwdArgs &A, hipStream_t s) {
 // pass B of the gather-mode backward (same instantiation set as the tiled pass A)
 int MA_CAT(launch_bwd_key_, MA_SUFFIX)(const BwdArgs &A, int CH, int R, hipStream_t s) {
     MA_KCASE(8) MA_KCASE(16) MA_KCASE(32) MA_KCASE(40) MA_KCASE(64)
-#if MA_DTYPE != 0
-    MA_KCASE(80) MA_KCASE(128)
-#endif
+    MA_KCASE(80) MA_KCASE(96) MA_KCASE(128) MA_KCASE(192)
     (void)A; (void)s;
     return -1;
 }

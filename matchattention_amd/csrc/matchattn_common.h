@@ -153,11 +153,14 @@ template <int CTRL> __device__ __forceinline__ float dpp_mov(float x) {
     return as_f32((uint32_t)__builtin_amdgcn_update_dpp(0, (int)as_u32(x), CTRL, 0xf, 0xf, false));
 }
 template <int LPH> __device__ __forceinline__ float group_sum(float x) {
-    static_assert(LPH == 1 || LPH == 2 || LPH == 4 || LPH == 8 || LPH == 16, "group size");
+    static_assert(LPH == 1 || LPH == 2 || LPH == 4 || LPH == 8 || LPH == 16 || LPH == 32 || LPH == 64, "group size");
     if (LPH >= 2) x += dpp_mov<0xB1>(x);   // quad_perm [1,0,3,2]
     if (LPH >= 4) x += dpp_mov<0x4E>(x);   // quad_perm [2,3,0,1]
     if (LPH >= 8) x += dpp_mov<0x141>(x);  // row_half_mirror
     if (LPH >= 16) x += dpp_mov<0x140>(x); // row_mirror
+    // (beyond a row of 16 lanes: through the LDS crossbar)
+    if (LPH >= 32) x += as_f32((uint32_t)__builtin_amdgcn_ds_bpermute((int)(((threadIdx.x & 63u) ^ 16u) * 4u), (int)as_u32(x)));
+    if (LPH >= 64) x += as_f32((uint32_t)__builtin_amdgcn_ds_bpermute((int)(((threadIdx.x & 63u) ^ 32u) * 4u), (int)as_u32(x)));
     return x;
 }
 

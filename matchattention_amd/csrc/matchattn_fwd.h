@@ -120,8 +120,8 @@ struct TiledCfg {
     static constexpr int EPV = Traits<T>::kEPV;
     static constexpr int NV = CH / EPV;                 // 16-byte vectors per head
     static constexpr int NVL = NV / VPL;                // lanes that carry data
-    static constexpr int LPH = NVL <= 1 ? 1 : NVL <= 2 ? 2 : NVL <= 4 ? 4 : NVL <= 8 ? 8 : 16;
-    static_assert(CH % EPV == 0 && NV % VPL == 0 && NVL <= 16, "unsupported head size for the tiled kernel");
+    static constexpr int LPH = NVL <= 1 ? 1 : NVL <= 2 ? 2 : NVL <= 4 ? 4 : NVL <= 8 ? 8 : NVL <= 16 ? 16 : NVL <= 32 ? 32 : 64;
+    static_assert(CH % EPV == 0 && NV % VPL == 0 && NVL <= 64, "unsupported head size for the tiled kernel");
     static constexpr int WN = 2 * R + 2;
     static constexpr int M = WN * WN;
     static constexpr int BLOCK = 256;

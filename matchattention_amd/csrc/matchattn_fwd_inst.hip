@@ -70,6 +70,12 @@ int MA_CAT(launch_fwd_tiled_, MA_SUFFIX)(const FwdArgs &A, int CH, int R, int VP
     MA_CASE(32, 1, 1) MA_CASE(32, 2, 1) MA_CASE(32, 1, 2) MA_CASE(32, 2, 2)
     MA_CASE(40, 1, 1) MA_CASE(40, 2, 1)
     MA_CASE(64, 1, 1) MA_CASE(64, 2, 1) MA_CASE(64, 1, 2) MA_CASE(64, 2, 2)
+    // (the coarse levels of the reference's `small` and `base` variants in its default precision: 20, 24 and 32 vectors
+    // per head, two per lane on 16 lanes)
+    MA_CASE(80, 1, 2) MA_CASE(80, 2, 2)
+    MA_CASE(96, 1, 2) MA_CASE(96, 2, 2)
+    MA_CASE(128, 1, 2) MA_CASE(128, 2, 2)
+    MA_CASE(192, 1, 2) MA_CASE(192, 2, 2)              // (24 lanes of 32 carry a head-query)
 #else
     // 16-bit types: 8 channels per 16-byte vector
     MA_CASE(8, 1, 1) MA_CASE(8, 2, 1)
@@ -78,7 +84,9 @@ int MA_CAT(launch_fwd_tiled_, MA_SUFFIX)(const FwdArgs &A, int CH, int R, int VP
     MA_CASE(40, 1, 1) MA_CASE(40, 2, 1)
     MA_CASE(64, 1, 1) MA_CASE(64, 2, 1) MA_CASE(64, 1, 2) MA_CASE(64, 2, 2)
     MA_CASE(80, 1, 1) MA_CASE(80, 2, 1)
+    MA_CASE(96, 1, 1) MA_CASE(96, 2, 1)
     MA_CASE(128, 1, 1) MA_CASE(128, 2, 1) MA_CASE(128, 1, 2) MA_CASE(128, 2, 2)
+    MA_CASE(192, 1, 2) MA_CASE(192, 2, 2)
 #endif
     (void)A; (void)s; (void)name;
     return -1;

@@ -68,6 +68,15 @@ MODEL_SHAPES = {
     for hw, c, r in ((48, 160, 2), (96, 128, 2), (192, 64, 1), (384, 32, 1)) for kind in ("cross", "self")
 }
 
+# The same frame through the `base` variant in the precision the reference's script defaults to (run_img.py:195-196,
+# models/convformer.py:372-380: channels 128, 256, 320, 512 from the finest level; fp32): heads of 32, 64, 80 and 128
+# channels.
+MODEL_SHAPES_BASE_F32 = {
+    f"base1536_{hw}x{hw}_c{c}_r{r}_{kind}": Workload(f"base1536_{hw}x{hw}_c{c}_r{r}_{kind}", torch.float32, 2, hw, hw, c, 4, r,
+                                                    f"stereo:{hw // 4}" if kind == "cross" else "gauss:2", kind == "self", True)
+    for hw, c, r in ((48, 512, 2), (96, 320, 2), (192, 256, 1), (384, 128, 1)) for kind in ("cross", "self")
+}
+
 
 def clamp_max_offset(max_offset: torch.Tensor, H: int, W: int, r: int) -> torch.Tensor:
     """The clamp the attention module applies before calling the operator
@@ -87,7 +96,9 @@ def make_inputs(wl: Workload, device="cuda", seed: Optional[int] = None, smooth:
     `rows` limits the map to its first rows (a bounded sample of the same workload)."""
     H = wl.H if rows is None else min(rows, wl.H)
     if seed is None:
-        seed = list(WORKLOADS).index(wl.name) if wl.name in WORKLOADS else 100 + list(MODEL_SHAPES).index(wl.name)
+        seed = (list(WORKLOADS).index(wl.name) if wl.name in WORKLOADS else
+                100 + list(MODEL_SHAPES).index(wl.name) if wl.name in MODEL_SHAPES else
+                200 + list(MODEL_SHAPES_BASE_F32).index(wl.name))
     g = torch.Generator(device=device).manual_seed(1000 + seed)
     N = H * wl.W
 

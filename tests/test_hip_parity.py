@@ -60,6 +60,18 @@ CASES = [
     (1, 10, 12, 3, 12, 1, torch.float16, "mixed", True),    # generic kernel
     (1, 12, 12, 4, 32, 2, torch.bfloat16, "mixed", True),
     (1, 12, 12, 2, 16, 1, torch.bfloat16, "stereo", True),
+    # the coarse levels of the reference's `small` and `base` variants in its default precision, and head sizes of its
+    # `large` configuration: more than 16 vectors per head (two per lane in the forward and the per-key pass, 32 lanes per
+    # head-query in the per-query pass)
+    (1, 9, 11, 2, 80, 2, torch.float32, "mixed", True),
+    (2, 8, 9, 1, 128, 2, torch.float32, "mixed", False),
+    (1, 10, 9, 2, 96, 1, torch.float32, "stereo", True),
+    (1, 9, 10, 2, 128, 1, torch.float32, "mixed", True),
+    (1, 9, 11, 2, 96, 2, torch.float16, "mixed", True),
+    (1, 8, 12, 1, 192, 2, torch.float16, "mixed", False),
+    (1, 9, 9, 2, 192, 1, torch.bfloat16, "stereo", True),
+    (1, 8, 9, 1, 192, 2, torch.float32, "mixed", True),
+    (1, 9, 8, 2, 192, 1, torch.float32, "mixed", False),
 ]
 
 
