@@ -627,6 +627,53 @@ def test_random_shapes_match_oracle(hip_lib, case):
     check_grads(got, mo, q, k, v, H, W, r, scale, d_out, d_attn, "random shapes bwd")
 
 
+def _big_head_cases(n=16, seed=4711):
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    while len(cases) < n:
+        dt = rnd.choice([torch.float32, torch.float32, torch.float16, torch.bfloat16])
+        Ch = rnd.choice([80, 96, 128, 192])
+        r = rnd.choice([1, 2])
+        h = rnd.choice([1, 2, 3, 4])
+        B = rnd.choice([1, 2])
+        H, W = rnd.randint(2 * r + 2, 14), rnd.randint(2 * r + 2, 18)
+        if B * H * W * h * Ch > 150_000:
+            continue
+        cases.append((B, H, W, h, Ch, r, dt, rnd.choice(["mixed", "stereo", "interior"]), rnd.random() < 0.6, rnd.random() < 0.6,
+                      rnd.choice([-1, 0, 2]), len(cases)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _big_head_cases(), ids=lambda c: f"{c[11]}_{str(c[6]).split('.')[1]}_B{c[0]}_{c[1]}x{c[2]}_h{c[3]}_ch{c[4]}_r{c[5]}_{c[7]}_bm{c[10]}")
+def test_heads_of_more_than_sixteen_vectors_match_oracle(hip_lib, case):
+    # heads of 80 to 192 channels (the coarse levels of the reference's larger variants): two vectors per lane in the
+    # forward and the per-key pass, 32 lanes per head-query in the per-query pass; seeded shapes with odd head counts
+    # and maps barely larger than the window, in every type and in the gathering and the scattering backward
+    from matchattention_amd import _cabi
+    B, H, W, h, Ch, r, dt, offs, clamp, per_head, bmode, idx = case
+    M = (2 * r + 2) ** 2
+    mo, q, k, v = make_case(B, H, W, h, Ch, r, dt, seed=900 + idx, offsets=offs, clamp=clamp, per_head=per_head)
+    scale = Ch ** -0.5
+    g = torch.Generator().manual_seed(idx)
+    d_out = torch.randn(B, H * W, h * Ch, generator=g).to(dt)
+    d_attn = torch.randn(B, H * W, h, M, generator=g).to(dt) if idx % 3 else None
+    want_out, want_attn = O.forward(mo, q, k, v, H, W, [r, r], scale)
+    dev = _dev(mo, q, k, v)
+    try:
+        _cabi.set_option("backward_mode", bmode)
+        out, attn = hip_forward(hip_lib, *dev, H, W, r, scale)
+        assert "generic" not in _cabi.last_forward_kernel(), _cabi.last_forward_kernel()
+        got = hip_backward(hip_lib, *dev, H, W, r, scale, d_out.cuda(), None if d_attn is None else d_attn.cuda())
+        assert "generic" not in _cabi.last_backward_kernel(), _cabi.last_backward_kernel()
+    finally:
+        _cabi.set_option("backward_mode", -1)
+    tol = TOL[dt]
+    assert torch.isfinite(out).all() and torch.isfinite(attn).all()
+    assert rel_err(attn.cpu(), want_attn) <= tol and rel_err(out.cpu(), want_out) <= tol
+    check_grads(got, mo, q, k, v, H, W, r, scale, d_out, d_attn, "big heads bwd")
+
+
 @pytest.mark.parametrize("tiles", [False, True])
 def test_fused_call_replays_from_a_hip_graph(hip_lib, tiles):
     # the fused entry point touches nothing on the host (on the LDS-tile path it adds one small kernel that writes the
