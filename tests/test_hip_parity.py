@@ -493,6 +493,9 @@ def _module_steps(rel, q, k, v, gate, H, W, r, h, attend):
     (torch.float32, 16, 4, 1, (2, 15, 22), True, True, ("forward_lds", -1)),
     (torch.bfloat16, 32, 2, 2, (1, 8, 300), True, True, ("forward_lds", -1)),    # x beyond bf16's exact integers
     (torch.float16, 32, 4, 2, (1, 17, 19), False, True, ("forward_variant", 0)),  # generic kernel
+    (torch.float16, 64, 4, 2, (2, 23, 41), True, True, ("forward_lds", 1)),      # LDS tiles, heads of 64 channels as two half-heads
+    (torch.bfloat16, 64, 2, 2, (1, 21, 40), False, True, ("forward_lds", 1)),
+    (torch.float32, 80, 2, 2, (1, 12, 20), True, True, ("forward_lds", -1)),     # two vectors per lane
 ])
 def test_fused_module_forward_is_bit_identical_to_the_separate_steps(hip_lib, dt, Ch, h, r, shape, shared, gated, opt):
     from matchattention_amd import _cabi, fused_module_forward
