@@ -226,7 +226,9 @@ def test_row_skip_does_not_change_results(hip_lib):
     ("mixed", True, True, 32, 2, (2, 6, 7, 2)), ("interior", False, True, 16, 1, (1, 8, 130, 4)),
     # one tile row 188 tiles wide; one tile column 313 tiles tall; three images whose last strip of tiles is 2 wide
     ("stereo", False, True, 16, 2, (1, 6, 3000, 4)), ("mixed", True, True, 32, 2, (1, 2500, 7, 2)),
-    ("mixed", False, True, 32, 2, (3, 20, 150, 2))])
+    ("mixed", False, True, 32, 2, (3, 20, 150, 2)),
+    # heads of 64 channels, an odd number of them, a position per head and a shared one (16-bit types: two half-heads of 32)
+    ("mixed", True, True, 64, 2, (2, 21, 37, 3)), ("stereo", False, True, 64, 2, (1, 30, 45, 1))])
 @pytest.mark.parametrize("dt", [torch.float16, torch.float32, torch.bfloat16], ids=["f16", "f32", "bf16"])
 def test_lds_tile_forward_matches_oracle(hip_lib, dt, offs, per_head, clamp, Ch, r, shape):
     # forward_lds=1: queries bucketed by K/V tile, every tap read from LDS; without the input clamp some
