@@ -1,19 +1,27 @@
-// Ordering of the queries by sampling target (gfx950).
+// Ordering of the queries by sampling target (gfx950): a counting sort whose bins are pixels, 8-column groups or
+// K/V tiles, depending on who asks.
 //
-// With spatially incoherent offsets, neighbouring queries gather from unrelated places and
-// every tap line misses L1.  The forward kernel may therefore walk the queries in the order of
-// a counting sort on coarse target bins (bin = batch item, target row, 8-column group): lanes
-// and wavefronts that run together then touch adjacent K/V lines.  The result of each query
-// does not depend on the order, so the output is unchanged.
+//   * the direct forward may walk the queries in the order of coarse target bins (batch item, target row, 8-column
+//     group) when the field is incoherent: lanes and wavefronts that run together then touch adjacent K/V lines;
+//   * the LDS-tile kernels take their work from buckets of one K/V tile each (optionally cut into sub-buckets by the
+//     row of the window inside the tile);
+//   * the backward's per-key pass follows an exact inverse index: one bin per target pixel, the entries of a bin in
+//     ascending pixel order (so that every sum runs in a fixed order), the window centres kept beside them.
+// The result of a query never depends on the order, so outputs do not change with it.
 //
-// Three small kernels fill perm[hd][slot] = pixel index:
-//   probe   : decides, on the device, whether the ordering is worth using (incoherent field)
-//             and whether every head of every pixel falls in head 0's bin (cross-attention:
-//             one offset shared by all heads, so one permutation serves all heads)
-//   count   : bin counts and the rank of each pixel within its bin (head 0; count_heads: the
-//             other heads, only when they need their own permutation)
-//   scan    : exclusive prefix sum of the bin counts of each counted head (two levels)
-//   scatter : perm[hd][start[bin] + rank] = pixel
+// Kernels, in stream order (perm[hd][slot] = pixel index is what they fill):
+//   probe         whether the ordering is worth using (incoherent field; skipped when it is not optional) and whether
+//                 every head of every pixel falls in head 0's bin (one offset shared by the heads: one order serves all)
+//   count         bin counts and the arrival rank of each pixel within its bin (a grid row per head; the rows of heads
+//                 1.. leave when the heads share head 0's order)
+//   rowscan,      exclusive prefix sums: the bins of a bin row by one wavefront, then the row totals
+//   rowtot_scan
+//   scatter       perm[hd][start[bin] + rank] = pixel (and its centre); by the way, the bucket populations the tile
+//                 work list is cut from
+//   bin_order,    exact index only: the entries of every bin into ascending pixel order (one thread per small bin, one
+//   big_bins_*    thread per entry of the large bins along the border)
+//   small         exact index of maps up to kSmallSortMaxN pixels: everything after the probe in one launch, one
+//                 workgroup per image and head
 #pragma once
 #include "matchattn_common.h"
 
