@@ -446,7 +446,7 @@ __global__ __launch_bounds__(256) void sort_big_bins_store_kernel(SortArgs S) {
 // limit is where one CU stops being faster than seven launches over the whole chip: a variant for images of up to
 // 40 448 pixels -- 16-bit counters, two per LDS word, the positions read three times -- took 90 us at 2 x 192 x 192
 // where the kernels above take 43.)
-constexpr int kSmallSortMaxN = 10240, kSmallSortThreads = 1024;
+constexpr int kSmallSortMaxN = 16384, kSmallSortThreads = 1024;
 template <int DT>
 __global__ __launch_bounds__(kSmallSortThreads) void sort_small_kernel(SortArgs S) {
     __shared__ int tab[kSmallSortMaxN];              // bin counts, then bin starts

@@ -156,9 +156,9 @@ def test_lds_tile_backward_matches_autograd(hip_lib, dt, offs, per_head, clamp, 
 
 
 @pytest.mark.parametrize("per_head", [True, False], ids=["per_head", "shared"])
-@pytest.mark.parametrize("shape", [(1, 100, 100), (1, 110, 100), (3, 30, 40)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", [(1, 127, 128), (1, 130, 130), (3, 30, 40)], ids=lambda s: "x".join(map(str, s)))
 def test_inverse_index_of_small_and_larger_maps(hip_lib, shape, per_head):
-    # The per-key pass follows an inverse index (which queries sample each pixel).  Maps of up to 10240 pixels get it
+    # The per-key pass follows an inverse index (which queries sample each pixel).  Maps of up to 16384 pixels get it
     # from one workgroup per image and head, larger ones from the chain of count, scan, scatter and ordering kernels:
     # a map on either side of that size and a batch of small ones, with unclamped offsets of which a good share lies
     # outside the map, so that the bins along the border hold hundreds of entries.  Gradients against the oracle's,
